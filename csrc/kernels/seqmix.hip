@@ -1,0 +1,603 @@
+// Sequence mixers and their glue for hybrid decoders (gfx950): Dynamic-Tanh norms over an fp32 residual stream,
+// paged softmax attention with a per-head sink term and separate key / value head sizes (prefill and decode),
+// partial rotary + value RMS norm + paged K/V store, linear attention with a fixed per-head decay and a carried
+// fp32 state, a minGRU scan with a carried fp32 state, a sigmoid-gated RMS norm and a clamped GLU.
+//
+// Precision: activations are bf16 or fp32 (dt: 0 = bf16, 1 = fp32; K/V caches hold the same type); the residual
+// stream, norms, attention scores / weights / accumulators, decays and recurrent states are fp32 in both.
+// Recurrent states start from zero when a sequence's first token of the launch is position 0 (no reset pass:
+// a freed and re-used state slot never leaks), and are loaded from / stored to the sequence's state slot.
+#include "common.h"
+
+GRAG_ERR_UNIT(seqmix)
+
+namespace grag {
+
+template <typename T> __device__ __forceinline__ float ldf(const T* p);
+template <> __device__ __forceinline__ float ldf<bf16>(const bf16* p) { return (float)*p; }
+template <> __device__ __forceinline__ float ldf<float>(const float* p) { return *p; }
+template <typename T> __device__ __forceinline__ void stf(T* p, float v);
+template <> __device__ __forceinline__ void stf<bf16>(bf16* p, float v) { *p = (bf16)v; }
+template <> __device__ __forceinline__ void stf<float>(float* p, float v) { *p = v; }
+
+__device__ __forceinline__ float sigmoidf_(float x) { return 1.f / (1.f + __expf(-x)); }
+__device__ __forceinline__ float sigmoid_acc(float x) { return 1.f / (1.f + expf(-x)); }
+__device__ __forceinline__ float silu_acc(float x) { return x / (1.f + expf(-x)); }
+
+// ------------------------------------------------------------------------------------------------ embedding
+template <typename T>
+__global__ void embed_f32_kernel(const int* __restrict__ ids, const T* __restrict__ table, float* __restrict__ out,
+                                 int H, int vocab) {
+  const int t = blockIdx.x;
+  const int id = ids[t];
+  if (!index_ok(id, vocab, ERR_EMBED_TOKEN)) {
+    for (int i = threadIdx.x; i < H; i += blockDim.x) out[(size_t)t * H + i] = 0.f;
+    return;
+  }
+  const T* row = table + (size_t)id * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) out[(size_t)t * H + i] = ldf(row + i);
+}
+
+// ------------------------------------------------------------------------------------------------ Dynamic Tanh
+// resid (fp32 [T, H], in place) += dyt1(y) + add_rows + add_vec   (each term optional), then
+// out = dyt2(resid) (optional).  dyt(x) = tanh(alpha x) w + b, no statistics.
+template <typename T>
+__global__ void dyt_residual_kernel(const T* __restrict__ y, float a1, const float* __restrict__ w1,
+                                    const float* __restrict__ b1, float* __restrict__ resid,
+                                    const float* __restrict__ add_rows, const float* __restrict__ add_vec, float a2,
+                                    const float* __restrict__ w2, const float* __restrict__ b2, T* __restrict__ out,
+                                    int H) {
+  const size_t base = (size_t)blockIdx.x * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    float x = resid[base + i];
+    if (y != nullptr) x += tanhf(a1 * ldf(y + base + i)) * w1[i] + b1[i];
+    if (add_rows != nullptr) x += add_rows[base + i];
+    if (add_vec != nullptr) x += add_vec[i];
+    if (y != nullptr || add_rows != nullptr || add_vec != nullptr) resid[base + i] = x;
+    if (out != nullptr) stf(out + base + i, tanhf(a2 * x) * w2[i] + b2[i]);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ rotary + K/V store
+// proj [T, ld]: q heads at column qoff (H x d), k heads at koff (G x d), v heads at voff (G x vd).
+// q_out [T, H*d] = rotated q; k_cache [nblk, G, BS, d] <- rotated k; v_cache [nblk, G, BS, vd] <- v / rms(v).
+// Rotation: the first rd dims of a head, dim i paired with i + rd/2; table row p = cos[0:rd/2] | sin[0:rd/2] (fp32).
+template <typename T>
+__global__ void rope_vnorm_store_kernel(const T* __restrict__ proj, int ld, int qoff, int koff, int voff,
+                                        const int* __restrict__ positions, const float* __restrict__ table,
+                                        int table_rows, const int* __restrict__ slot_mapping, T* __restrict__ q_out,
+                                        T* __restrict__ k_cache, T* __restrict__ v_cache, int H, int G, int d, int vd,
+                                        int rd, int BS, long nslots, float eps) {
+  const int t = blockIdx.x;
+  const T* row = proj + (size_t)t * ld;
+  const int pos = positions[t];
+  const bool pos_ok = rd == 0 || index_ok(pos, table_rows, ERR_ROPE_POS);
+  const float* cs = table + (size_t)(pos_ok ? pos : 0) * rd;
+  const int half = rd >> 1;
+  const int slot = slot_mapping[t];
+  const bool store = slot >= 0 && index_ok(slot, nslots, ERR_KV_SLOT);
+  const int blk = store ? slot / BS : 0, off = store ? slot % BS : 0;
+  const int nq = H * d, nk = G * d;
+  for (int e = threadIdx.x; e < nq + nk; e += blockDim.x) {
+    const bool isq = e < nq;
+    const int f = isq ? e : e - nq;
+    const int hh = f / d, i = f - hh * d;
+    const T* x = row + (isq ? qoff : koff) + hh * d;
+    float v = ldf(x + i);
+    if (i < rd && pos_ok) {
+      if (i < half) {
+        v = v * cs[i] - ldf(x + i + half) * cs[half + i];
+      } else {
+        const int j = i - half;
+        v = v * cs[j] + ldf(x + j) * cs[half + j];
+      }
+    }
+    if (isq) {
+      stf(q_out + (size_t)t * nq + e, v);
+    } else if (store) {
+      stf(k_cache + (((size_t)blk * G + hh) * BS + off) * d + i, v);
+    }
+  }
+  // values: one wave per kv head, RMS over vd in fp32
+  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  for (int g = wid; g < G; g += nw) {
+    const T* x = row + voff + g * vd;
+    float ss = 0.f;
+    for (int i = lane; i < vd; i += 64) {
+      const float v = ldf(x + i);
+      ss += v * v;
+    }
+    ss = wave_sum(ss);
+    const float r = 1.f / sqrtf(ss / (float)vd + eps);
+    if (store)
+      for (int i = lane; i < vd; i += 64) stf(v_cache + (((size_t)blk * G + g) * BS + off) * vd + i, ldf(x + i) * r);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ sink attention
+// softmax over the visible keys plus one key-less, value-less term exp(sink_h) in the denominator: the running
+// (max, sum) starts at (sink_h, 1) instead of (-inf, 0).
+constexpr int SA_NQ = 4;   // queries per wave (prefill)
+constexpr int SA_VC = 4;   // 64-wide value-dim chunks per lane: vd <= 256
+
+// prefill: grid (q tiles of 4 waves x SA_NQ queries, H, nseq), 256 threads.  A tile of KT keys (K [KT][d+1] and
+// V [KT][vd], fp32) is staged in LDS per step; lane = key for the scores, lane = value dim for the output.
+template <typename T>
+__global__ void __launch_bounds__(256)
+sink_attn_prefill_kernel(const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+                         T* __restrict__ out, int out_ld, const int* __restrict__ block_tables, int bt_stride,
+                         const int* __restrict__ q_start, const int* __restrict__ ctx_len,
+                         const float* __restrict__ sinks, int H, int G, int d, int vd, int BS, float scale,
+                         float out_scale, int KT, int nblocks) {
+  extern __shared__ float smem[];
+  const int QT = 4 * SA_NQ;
+  const int seq = blockIdx.z, h = blockIdx.y, g = h / (H / G);
+  const int qa = q_start[seq], qlen = q_start[seq + 1] - qa, ctx = ctx_len[seq];
+  const int q0 = blockIdx.x * QT;
+  if (q0 >= qlen) return;
+  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+  const int dp = d + 1;
+  float* Ks = smem;                    // [KT][d+1]
+  float* Vs = Ks + KT * dp;            // [KT][vd]
+  float* Qs = Vs + KT * vd;            // [QT][d]
+  float* Ps = Qs + QT * d;             // [4 waves][SA_NQ][64]
+  for (int idx = threadIdx.x; idx < QT * d; idx += 256) {
+    const int qi = idx / d, i = idx - qi * d;
+    const int tq = q0 + qi;
+    Qs[idx] = tq < qlen ? ldf(q + ((size_t)(qa + tq) * H + h) * d + i) : 0.f;
+  }
+  const int pos0 = ctx - qlen;  // position of the launch's first query of this sequence
+  float m[SA_NQ], l[SA_NQ], acc[SA_NQ][SA_VC];
+  const float sink = sinks[h];
+#pragma unroll
+  for (int n = 0; n < SA_NQ; ++n) {
+    m[n] = sink;
+    l[n] = 1.f;
+#pragma unroll
+    for (int c = 0; c < SA_VC; ++c) acc[n][c] = 0.f;
+  }
+  const int last_q = min(q0 + QT, qlen) - 1;
+  const int nkeys = min(ctx, pos0 + last_q + 1);
+  const int* bt = block_tables + (size_t)seq * bt_stride;
+  for (int k0 = 0; k0 < nkeys; k0 += KT) {
+    __syncthreads();
+    const int kn = min(KT, nkeys - k0);
+    for (int idx = threadIdx.x; idx < kn * d; idx += 256) {
+      const int kk = idx / d, i = idx - kk * d;
+      const int key = k0 + kk;
+      const int blk = bt[key / BS];
+      float v = 0.f;
+      if (index_ok(blk, nblocks, ERR_BLOCK_PREFILL))
+        v = ldf(k_cache + (((size_t)blk * G + g) * BS + key % BS) * d + i);
+      Ks[kk * dp + i] = v;
+    }
+    for (int idx = threadIdx.x; idx < kn * vd; idx += 256) {
+      const int kk = idx / vd, i = idx - kk * vd;
+      const int key = k0 + kk;
+      const int blk = bt[key / BS];
+      float v = 0.f;
+      if (blk >= 0 && blk < nblocks) v = ldf(v_cache + (((size_t)blk * G + g) * BS + key % BS) * vd + i);
+      Vs[kk * vd + i] = v;
+    }
+    __syncthreads();
+    // scores: lane = key
+    float s[SA_NQ];
+#pragma unroll
+    for (int n = 0; n < SA_NQ; ++n) s[n] = 0.f;
+    if (lane < kn) {
+      const float* kr = Ks + lane * dp;
+      const float* qr = Qs + (wid * SA_NQ) * d;
+      for (int i = 0; i < d; ++i) {
+        const float kv = kr[i];
+#pragma unroll
+        for (int n = 0; n < SA_NQ; ++n) s[n] = fmaf(qr[n * d + i], kv, s[n]);
+      }
+    }
+    float* pw = Ps + wid * SA_NQ * 64;
+#pragma unroll
+    for (int n = 0; n < SA_NQ; ++n) {
+      const int tq = q0 + wid * SA_NQ + n;
+      const bool vis = lane < kn && tq < qlen && (k0 + lane) <= pos0 + tq;
+      const float sc = vis ? s[n] * scale : -INFINITY;
+      const float mn = fmaxf(m[n], wave_max(sc));
+      const float p = vis ? expf(sc - mn) : 0.f;
+      const float alpha = expf(m[n] - mn);
+      l[n] = l[n] * alpha + wave_sum(p);
+      m[n] = mn;
+#pragma unroll
+      for (int c = 0; c < SA_VC; ++c) acc[n][c] *= alpha;
+      pw[n * 64 + lane] = p;
+    }
+    // (the wave's own LDS rows: a wave-level fence is enough)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+#pragma unroll
+    for (int c = 0; c < SA_VC; ++c) {
+      const int j = lane + 64 * c;
+      if (j < vd) {
+        for (int kk = 0; kk < kn; ++kk) {
+          const float vv = Vs[kk * vd + j];
+#pragma unroll
+          for (int n = 0; n < SA_NQ; ++n) acc[n][c] = fmaf(pw[n * 64 + kk], vv, acc[n][c]);
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int n = 0; n < SA_NQ; ++n) {
+    const int tq = q0 + wid * SA_NQ + n;
+    if (tq >= qlen) continue;
+    const float r = out_scale / l[n];
+#pragma unroll
+    for (int c = 0; c < SA_VC; ++c) {
+      const int j = lane + 64 * c;
+      if (j < vd) stf(out + (size_t)(qa + tq) * out_ld + h * vd + j, acc[n][c] * r);
+    }
+  }
+}
+
+// decode (one query token per sequence): grid (H, nseq), 256 threads.  Each of the 4 waves walks every 4th
+// 64-key tile (lane = key, K rows read from the cache), keeps its own (m, l, acc); the waves merge through LDS.
+template <typename T>
+__global__ void __launch_bounds__(256)
+sink_attn_decode_kernel(const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+                        T* __restrict__ out, int out_ld, const int* __restrict__ block_tables, int bt_stride,
+                        const int* __restrict__ ctx_len, const float* __restrict__ sinks, int H, int G, int d, int vd,
+                        int BS, float scale, float out_scale, int nblocks) {
+  extern __shared__ float smem[];
+  const int seq = blockIdx.y, h = blockIdx.x, g = h / (H / G);
+  const int ctx = ctx_len[seq];
+  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+  float* Qs = smem;               // [d]
+  float* Ps = Qs + d;             // [4][64]
+  float* Ms = Ps + 4 * 64;        // [4] m, [4] l
+  float* As = Ms + 8;             // [4][vd]
+  for (int i = threadIdx.x; i < d; i += 256) Qs[i] = ldf(q + ((size_t)seq * H + h) * d + i);
+  __syncthreads();
+  float m = wid == 0 ? sinks[h] : -INFINITY, l = wid == 0 ? 1.f : 0.f;
+  float acc[SA_VC];
+#pragma unroll
+  for (int c = 0; c < SA_VC; ++c) acc[c] = 0.f;
+  const int* bt = block_tables + (size_t)seq * bt_stride;
+  float* pw = Ps + wid * 64;
+  const int ntiles = (ctx + 63) >> 6;
+  for (int t = wid; t < ntiles; t += 4) {
+    const int key = t * 64 + lane;
+    const bool vis = key < ctx;
+    float s = 0.f;
+    int blk = 0;
+    if (vis) {
+      blk = bt[key / BS];
+      if (!index_ok(blk, nblocks, ERR_BLOCK_DECODE)) blk = 0;
+      const T* kr = k_cache + (((size_t)blk * G + g) * BS + key % BS) * d;
+      for (int i = 0; i < d; ++i) s = fmaf(Qs[i], ldf(kr + i), s);
+    }
+    const float sc = vis ? s * scale : -INFINITY;
+    const float mn = fmaxf(m, wave_max(sc));  // (wave 0 always has the finite sink; others see >= 1 visible key)
+    const float p = vis ? expf(sc - mn) : 0.f;
+    const float alpha = (m == -INFINITY) ? 0.f : expf(m - mn);
+    l = l * alpha + wave_sum(p);
+    m = mn;
+    pw[lane] = p;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    const int kn = min(64, ctx - t * 64);
+#pragma unroll
+    for (int c = 0; c < SA_VC; ++c) {
+      const int j = lane + 64 * c;
+      float a = acc[c] * alpha;
+      if (j < vd) {
+        for (int kk = 0; kk < kn; ++kk) {
+          const int key2 = t * 64 + kk;
+          int b2 = bt[key2 / BS];
+          if (b2 < 0 || b2 >= nblocks) b2 = 0;
+          a = fmaf(pw[kk], ldf(v_cache + (((size_t)b2 * G + g) * BS + key2 % BS) * vd + j), a);
+        }
+      }
+      acc[c] = a;
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+  if (lane == 0) {
+    Ms[wid] = m;
+    Ms[4 + wid] = l;
+  }
+#pragma unroll
+  for (int c = 0; c < SA_VC; ++c) {
+    const int j = lane + 64 * c;
+    if (j < vd) As[wid * vd + j] = acc[c];
+  }
+  __syncthreads();
+  if (wid == 0) {
+    float M = Ms[0];
+    for (int w = 1; w < 4; ++w) M = fmaxf(M, Ms[w]);
+    float L = 0.f, f[4];
+    for (int w = 0; w < 4; ++w) {
+      f[w] = Ms[w] == -INFINITY ? 0.f : expf(Ms[w] - M);
+      L += Ms[4 + w] * f[w];
+    }
+    const float r = out_scale / L;
+#pragma unroll
+    for (int c = 0; c < SA_VC; ++c) {
+      const int j = lane + 64 * c;
+      if (j < vd) {
+        float o = 0.f;
+        for (int w = 0; w < 4; ++w) o += As[w * vd + j] * f[w];
+        stf(out + (size_t)seq * out_ld + h * vd + j, o * r);
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ decay linear attention
+// Per head: S_t = decay_h S_(t-1) + k_t v_t^T, o_t = S_t^T q_t, with q, k, v = silu(projection) and S [d, vd] fp32.
+// grid (H, nseq); thread j < vd owns column j of S in registers (DMAX rows).  Tokens of the launch are walked in
+// order, TB at a time through LDS.  Serves prefill chunks (qlen tokens) and decode rows (qlen = 1) alike.
+template <typename T, int DMAX>
+__global__ void decay_attn_scan_kernel(const T* __restrict__ proj, int ld, int qoff, int koff, int voff,
+                                       const float* __restrict__ decay, float* __restrict__ state,
+                                       const int* __restrict__ slots, const int* __restrict__ q_start,
+                                       const int* __restrict__ ctx_len, float* __restrict__ out, int H, int d, int vd,
+                                       int nslots) {
+  constexpr int TB = 16;
+  extern __shared__ float smem[];  // [TB][2][d]
+  const int seq = blockIdx.y, h = blockIdx.x;
+  const int qa = q_start[seq], qlen = q_start[seq + 1] - qa;
+  if (qlen <= 0) return;
+  const int j = threadIdx.x;
+  const bool fresh = ctx_len[seq] - qlen == 0;
+  const int slot = slots[seq];
+  const bool slot_ok = index_ok(slot, nslots, ERR_SAMPLER_SLOT);
+  float* Sg = state + (((size_t)(slot_ok ? slot : 0) * H + h) * d) * vd;
+  const float lam = decay[h];
+  float S[DMAX];
+#pragma unroll
+  for (int i = 0; i < DMAX; ++i) S[i] = (!fresh && slot_ok && i < d && j < vd) ? Sg[(size_t)i * vd + j] : 0.f;
+  for (int t0 = 0; t0 < qlen; t0 += TB) {
+    const int nb = min(TB, qlen - t0);
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < nb * 2 * d; idx += blockDim.x) {
+      const int tt = idx / (2 * d), r = idx - tt * 2 * d;
+      const int which = r / d, i = r - which * d;
+      const T* row = proj + (size_t)(qa + t0 + tt) * ld + (which ? koff : qoff) + h * d;
+      smem[idx] = silu_acc(ldf(row + i));
+    }
+    __syncthreads();
+    if (j < vd) {
+      for (int tt = 0; tt < nb; ++tt) {
+        const size_t tok = (size_t)(qa + t0 + tt);
+        const float vj = silu_acc(ldf(proj + tok * ld + voff + h * vd + j));
+        const float* qs = smem + tt * 2 * d;
+        const float* ks = qs + d;
+        float o = 0.f;
+#pragma unroll
+        for (int i = 0; i < DMAX; ++i) {
+          if (i < d) {
+            S[i] = fmaf(lam, S[i], ks[i] * vj);
+            o = fmaf(S[i], qs[i], o);
+          }
+        }
+        out[tok * (size_t)(H * vd) + h * vd + j] = o;
+      }
+    }
+  }
+  if (slot_ok && j < vd) {
+#pragma unroll
+    for (int i = 0; i < DMAX; ++i)
+      if (i < d) Sg[(size_t)i * vd + j] = S[i];
+  }
+}
+
+// out [T, out_ld slice] = out_scale * x / rms(x) * w * sigmoid(gate), x fp32 [T, N]; gate at proj column goff.
+template <typename T>
+__global__ void gated_rmsnorm_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                     const T* __restrict__ proj, int ld, int goff, T* __restrict__ out, int out_ld,
+                                     int N, float eps, float out_scale) {
+  __shared__ float red[16];
+  const int t = blockIdx.x;
+  const float* xr = x + (size_t)t * N;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < N; i += blockDim.x) ss += xr[i] * xr[i];
+  ss = block_sum(ss, red);
+  const float r = out_scale / sqrtf(ss / (float)N + eps);
+  for (int i = threadIdx.x; i < N; i += blockDim.x) {
+    const float gt = sigmoid_acc(ldf(proj + (size_t)t * ld + goff + i));
+    stf(out + (size_t)t * out_ld + i, xr[i] * r * w[i] * gt);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ minGRU
+// z = sigmoid(pz + bz), u = px + bx, c = u >= 0 ? u + 1/2 : sigmoid(u); S_t = (1 - z) S_(t-1) + z c;
+// out = S_t * silu(pg).  grid (ceil(W / 256), nseq): one thread per channel walks the launch's tokens in order.
+template <typename T>
+__global__ void mingru_scan_kernel(const T* __restrict__ proj, int ld, int zoff, int xoff, int goff,
+                                   const float* __restrict__ bz, const float* __restrict__ bx,
+                                   float* __restrict__ state, const int* __restrict__ slots,
+                                   const int* __restrict__ q_start, const int* __restrict__ ctx_len,
+                                   T* __restrict__ out, int W, int nslots) {
+  const int seq = blockIdx.y;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  const int qa = q_start[seq], qlen = q_start[seq + 1] - qa;
+  if (c >= W || qlen <= 0) return;
+  const int slot = slots[seq];
+  const bool slot_ok = index_ok(slot, nslots, ERR_SAMPLER_SLOT);
+  float* sp = state + (size_t)(slot_ok ? slot : 0) * W + c;
+  float S = (ctx_len[seq] - qlen == 0 || !slot_ok) ? 0.f : *sp;
+  const float zb = bz[c], xb = bx[c];
+  for (int t = 0; t < qlen; ++t) {
+    const T* row = proj + (size_t)(qa + t) * ld;
+    const float z = sigmoid_acc(ldf(row + zoff + c) + zb);
+    const float u = ldf(row + xoff + c) + xb;
+    const float cand = u >= 0.f ? u + 0.5f : sigmoid_acc(u);
+    S = (1.f - z) * S + z * cand;
+    stf(out + (size_t)(qa + t) * W + c, S * silu_acc(ldf(row + goff + c)));
+  }
+  if (slot_ok) *sp = S;
+}
+
+// ------------------------------------------------------------------------------------------------ clamped GLU
+// gu [T, 2F] (gate | up): y = g sigmoid(alpha g) (u + 1), g = min(gate, limit), u = clamp(up, -limit, limit).
+template <typename T>
+__global__ void clamped_glu_kernel(const T* __restrict__ gu, T* __restrict__ out, int F, float limit, float alpha) {
+  const size_t t = blockIdx.y;
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= F) return;
+  const float g = fminf(ldf(gu + t * 2 * F + i), limit);
+  const float u = fminf(fmaxf(ldf(gu + t * 2 * F + F + i), -limit), limit);
+  stf(out + t * F + i, g * sigmoid_acc(alpha * g) * (u + 1.f));
+}
+
+}  // namespace grag
+
+using namespace grag;
+
+#define DT_DISPATCH(dt, ...)                   \
+  if ((dt) == 0) {                             \
+    using T = bf16;                            \
+    __VA_ARGS__                                \
+  } else {                                     \
+    using T = float;                           \
+    __VA_ARGS__                                \
+  }
+
+GRAG_API hipError_t grag_embed_f32(const int* ids, const void* table, float* out, int T_, int H, int vocab, int dt,
+                                   hipStream_t st) {
+  if (T_ <= 0) return hipSuccess;
+  DT_DISPATCH(dt, hipLaunchKernelGGL(embed_f32_kernel<T>, dim3(T_), dim3(256), 0, st, ids, (const T*)table, out, H,
+                                     vocab);)
+  return hipGetLastError();
+}
+
+GRAG_API hipError_t grag_dyt_residual(const void* y, float a1, const float* w1, const float* b1, float* resid,
+                                      const float* add_rows, const float* add_vec, float a2, const float* w2,
+                                      const float* b2, void* out, int T_, int H, int dt, hipStream_t st) {
+  if (T_ <= 0) return hipSuccess;
+  DT_DISPATCH(dt, hipLaunchKernelGGL(dyt_residual_kernel<T>, dim3(T_), dim3(256), 0, st, (const T*)y, a1, w1, b1,
+                                     resid, add_rows, add_vec, a2, w2, b2, (T*)out, H);)
+  return hipGetLastError();
+}
+
+GRAG_API hipError_t grag_rope_vnorm_store(const void* proj, int ld, int qoff, int koff, int voff, const int* positions,
+                                          const float* table, int table_rows, const int* slot_mapping, void* q_out,
+                                          void* k_cache, void* v_cache, int T_, int H, int G, int d, int vd, int rd,
+                                          int BS, long nslots, float eps, int dt, hipStream_t st) {
+  if (T_ <= 0) return hipSuccess;
+  DT_DISPATCH(dt, hipLaunchKernelGGL(rope_vnorm_store_kernel<T>, dim3(T_), dim3(256), 0, st, (const T*)proj, ld, qoff,
+                                     koff, voff, positions, table, table_rows, slot_mapping, (T*)q_out, (T*)k_cache,
+                                     (T*)v_cache, H, G, d, vd, rd, BS, nslots, eps);)
+  return hipGetLastError();
+}
+
+static int sa_key_tile(int d, int vd, size_t* bytes) {
+  // K [KT][d+1] + V [KT][vd] + Q [16][d] + P [4][SA_NQ][64], fp32; the largest tile of 64 / 32 / 16 keys under 144 KB
+  for (int kt = 64; kt >= 16; kt >>= 1) {
+    const size_t b = ((size_t)kt * (d + 1 + vd) + 16 * (size_t)d + 4 * SA_NQ * 64) * sizeof(float);
+    if (b <= 144 * 1024 || kt == 16) {
+      *bytes = b;
+      return kt;
+    }
+  }
+  return 16;
+}
+
+GRAG_API hipError_t grag_sink_attn_prefill(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                           int out_ld, const int* block_tables, int bt_stride, const int* q_start,
+                                           const int* ctx_len, const float* sinks, int nseq, int max_q_len, int H,
+                                           int G, int d, int vd, int BS, float scale, float out_scale, int nblocks,
+                                           int dt, hipStream_t st) {
+  if (nseq <= 0 || max_q_len <= 0) return hipSuccess;
+  if (vd > 64 * SA_VC || G <= 0 || H % G) return hipErrorInvalidValue;
+  size_t bytes;
+  const int KT = sa_key_tile(d, vd, &bytes);
+  if (bytes > 160 * 1024) return hipErrorInvalidValue;
+  const dim3 grid((max_q_len + 4 * SA_NQ - 1) / (4 * SA_NQ), H, nseq);
+  DT_DISPATCH(dt, {
+    if (bytes > 48 * 1024) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&sink_attn_prefill_kernel<T>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+      if (e != hipSuccess) return e;
+    }
+    hipLaunchKernelGGL(sink_attn_prefill_kernel<T>, grid, dim3(256), bytes, st, (const T*)q, (const T*)k_cache,
+                       (const T*)v_cache, (T*)out, out_ld, block_tables, bt_stride, q_start, ctx_len, sinks, H, G, d,
+                       vd, BS, scale, out_scale, KT, nblocks);
+  })
+  return hipGetLastError();
+}
+
+GRAG_API hipError_t grag_sink_attn_decode(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                          int out_ld, const int* block_tables, int bt_stride, const int* ctx_len,
+                                          const float* sinks, int nseq, int H, int G, int d, int vd, int BS,
+                                          float scale, float out_scale, int nblocks, int dt, hipStream_t st) {
+  if (nseq <= 0) return hipSuccess;
+  if (vd > 64 * SA_VC || G <= 0 || H % G) return hipErrorInvalidValue;
+  const size_t bytes = ((size_t)d + 4 * 64 + 8 + 4 * (size_t)vd) * sizeof(float);
+  DT_DISPATCH(dt, hipLaunchKernelGGL(sink_attn_decode_kernel<T>, dim3(H, nseq), dim3(256), bytes, st, (const T*)q,
+                                     (const T*)k_cache, (const T*)v_cache, (T*)out, out_ld, block_tables, bt_stride,
+                                     ctx_len, sinks, H, G, d, vd, BS, scale, out_scale, nblocks);)
+  return hipGetLastError();
+}
+
+template <typename T>
+static hipError_t launch_decay_scan(const T* proj, int ld, int qoff, int koff, int voff, const float* decay,
+                                    float* state, const int* slots, const int* q_start, const int* ctx_len, float* out,
+                                    int nseq, int H, int d, int vd, int nslots, hipStream_t st) {
+  const int threads = ((vd + 63) / 64) * 64;
+  const size_t bytes = (size_t)16 * 2 * d * sizeof(float);
+  const dim3 grid(H, nseq);
+#define DECAY_LAUNCH(DM)                                                                                          \
+  hipLaunchKernelGGL((decay_attn_scan_kernel<T, DM>), grid, dim3(threads), bytes, st, proj, ld, qoff, koff, voff, \
+                     decay, state, slots, q_start, ctx_len, out, H, d, vd, nslots)
+  if (d <= 16) {
+    DECAY_LAUNCH(16);
+  } else if (d <= 32) {
+    DECAY_LAUNCH(32);
+  } else if (d <= 64) {
+    DECAY_LAUNCH(64);
+  } else if (d <= 128) {
+    DECAY_LAUNCH(128);
+  } else {
+    DECAY_LAUNCH(256);
+  }
+#undef DECAY_LAUNCH
+  return hipGetLastError();
+}
+
+GRAG_API hipError_t grag_decay_attn_scan(const void* proj, int ld, int qoff, int koff, int voff, const float* decay,
+                                         float* state, const int* slots, const int* q_start, const int* ctx_len,
+                                         float* out, int nseq, int H, int d, int vd, int nslots, int dt,
+                                         hipStream_t st) {
+  if (nseq <= 0) return hipSuccess;
+  if (d > 256 || vd > 1024) return hipErrorInvalidValue;
+  DT_DISPATCH(dt, return launch_decay_scan<T>((const T*)proj, ld, qoff, koff, voff, decay, state, slots, q_start,
+                                              ctx_len, out, nseq, H, d, vd, nslots, st);)
+}
+
+GRAG_API hipError_t grag_gated_rmsnorm(const float* x, const float* w, const void* proj, int ld, int goff, void* out,
+                                       int out_ld, int T_, int N, float eps, float out_scale, int dt, hipStream_t st) {
+  if (T_ <= 0) return hipSuccess;
+  DT_DISPATCH(dt, hipLaunchKernelGGL(gated_rmsnorm_kernel<T>, dim3(T_), dim3(256), 0, st, x, w, (const T*)proj, ld,
+                                     goff, (T*)out, out_ld, N, eps, out_scale);)
+  return hipGetLastError();
+}
+
+GRAG_API hipError_t grag_mingru_scan(const void* proj, int ld, int zoff, int xoff, int goff, const float* bz,
+                                     const float* bx, float* state, const int* slots, const int* q_start,
+                                     const int* ctx_len, void* out, int nseq, int W, int nslots, int dt,
+                                     hipStream_t st) {
+  if (nseq <= 0) return hipSuccess;
+  const dim3 grid((W + 255) / 256, nseq);
+  DT_DISPATCH(dt, hipLaunchKernelGGL(mingru_scan_kernel<T>, grid, dim3(256), 0, st, (const T*)proj, ld, zoff, xoff,
+                                     goff, bz, bx, state, slots, q_start, ctx_len, (T*)out, W, nslots);)
+  return hipGetLastError();
+}
+
+GRAG_API hipError_t grag_clamped_glu(const void* gu, void* out, int T_, int F, float limit, float alpha, int dt,
+                                     hipStream_t st) {
+  if (T_ <= 0) return hipSuccess;
+  const dim3 grid((F + 255) / 256, T_);
+  DT_DISPATCH(dt, hipLaunchKernelGGL(clamped_glu_kernel<T>, grid, dim3(256), 0, st, (const T*)gu, (T*)out, F, limit,
+                                     alpha);)
+  return hipGetLastError();
+}

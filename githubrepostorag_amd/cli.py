@@ -18,6 +18,10 @@ engine, encoder, index, job workers and API together:
   ingest   ingest repositories (github | local dir | synthetic) into the
            index and optionally snapshot it to INDEX_DIR.
   ask      one RAG query through the agent, printing events as they arrive.
+  generate complete token-id prompts with a checkpoint directory's decoder (any served family) through the
+           engine's scheduler and sampler; prints one JSON line per prompt.
+  trace    replay a recorded token schedule (JSON steps on stdin) through the engine and write the logits it
+           asks for (engine/trace.py; bin/trace_run is this command).
   build    compile the gfx950 kernel library and the host runtime in-tree.
   config   print the resolved settings (env-compatible with the reference).
   bench    forward to bench.py (driver contract).
@@ -311,6 +315,32 @@ def cmd_bench(args, rest) -> int:
     return subprocess.call([sys.executable, os.path.join(root, "bench.py"), *rest])
 
 
+def cmd_trace(args) -> int:
+    from .engine.trace import run_trace
+
+    return run_trace(args.model, args.dtype, args.out, args.max_tokens, device=args.device, block_size=args.block_size)
+
+
+def cmd_generate(args) -> int:
+    import torch
+
+    from .engine.llm_engine import EngineConfig, LLMEngine
+    from .engine.sequence import SamplingParams
+    from .models import load_decoder
+
+    dev = args.device or ("cuda" if torch.cuda.is_available() else "cpu")
+    model = load_decoder(args.model, device=dev, dtype={"bfloat16": torch.bfloat16, "float32": torch.float32}[args.dtype])
+    prompts = [[int(t) for t in p.split(",") if t.strip()] for p in args.prompt_ids]
+    longest = max(len(p) for p in prompts) + args.max_tokens + 1
+    eng = LLMEngine(model, None, EngineConfig(max_num_seqs=max(1, min(len(prompts), 64)), max_model_len=longest,
+                                              num_blocks=len(prompts) * (-(-longest // 16) + 1) + 1))
+    sp = SamplingParams(max_tokens=args.max_tokens, temperature=args.temperature, top_p=args.top_p, top_k=args.top_k,
+                        ignore_eos=True, seed=args.seed)
+    for p, c in zip(prompts, eng.generate(prompts, sp)):
+        print(json.dumps({"prompt_ids": p, "token_ids": c.token_ids, "finish_reason": c.finish_reason}))
+    return 0
+
+
 def build_parser() -> argparse.ArgumentParser:
     ap = argparse.ArgumentParser(prog="githubrepostorag_amd", description=__doc__.split("\n\n")[0])
     sub = ap.add_subparsers(dest="cmd", required=True)
@@ -355,6 +385,24 @@ def build_parser() -> argparse.ArgumentParser:
     p = sub.add_parser("build", help="compile the native libraries in-tree")
     p.add_argument("--force", action="store_true")
     p.add_argument("-v", "--verbose", action="store_true")
+    p = sub.add_parser("trace", help="replay a token schedule from stdin, write the logits it asks for")
+    p.add_argument("--model", required=True, help="directory with config.json and model.safetensors")
+    p.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
+    p.add_argument("--out", required=True, help="directory for <step>.f32")
+    p.add_argument("--max-tokens", dest="max_tokens", type=int, required=True,
+                   help="tokens the live requests hold at most (sizes the KV pool)")
+    p.add_argument("--device")
+    p.add_argument("--block-size", dest="block_size", type=int, default=16)
+    p = sub.add_parser("generate", help="complete token-id prompts with a checkpoint directory's decoder")
+    p.add_argument("--model", required=True)
+    p.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
+    p.add_argument("--prompt-ids", dest="prompt_ids", nargs="+", required=True, help="comma-separated token ids")
+    p.add_argument("--max-tokens", dest="max_tokens", type=int, default=16)
+    p.add_argument("--temperature", type=float, default=0.0)
+    p.add_argument("--top-p", dest="top_p", type=float, default=1.0)
+    p.add_argument("--top-k", dest="top_k", type=int, default=0)
+    p.add_argument("--seed", type=int, default=None)
+    p.add_argument("--device")
     p = sub.add_parser("config", help="print resolved settings")
     common(p)
     sub.add_parser("bench", help="run bench.py (remaining args are forwarded)", add_help=False)
@@ -368,7 +416,7 @@ def main(argv=None) -> int:
         return cmd_bench(None, argv[1:])
     args = ap.parse_args(argv)
     return {"serve": cmd_serve, "replica": cmd_replica, "ingest": cmd_ingest, "ask": cmd_ask, "build": cmd_build,
-            "config": cmd_config}[args.cmd](args)
+            "config": cmd_config, "trace": cmd_trace, "generate": cmd_generate}[args.cmd](args)
 
 
 if __name__ == "__main__":

@@ -172,9 +172,19 @@ class LLMEngine:
         cfg = self.cfg
         cfg.max_model_len = min(cfg.max_model_len, model.cfg.max_position)
         bs = cfg.block_size
+        # models with recurrent state (has_state): a cached prompt prefix holds K/V but no state to resume from, so
+        # prefixes are never shared; the state pools are indexed by the scheduler's sequence slots (one more for
+        # the padding rows of captured batches)
+        self.has_state = bool(getattr(model, "has_state", False))
+        if self.has_state:
+            cfg.enable_prefix_caching = False
+            cfg.cascade_decode = False
+        if hasattr(model, "prepare"):
+            model.prepare(cfg.max_model_len)
         nblocks = cfg.num_blocks or self._plan_blocks()
         self.kv = KVCacheManager(nblocks, bs, cfg.enable_prefix_caching)
         self.kv_caches = model.allocate_kv_cache(nblocks, bs)
+        self.state = model.allocate_state(cfg.max_num_seqs + 1) if self.has_state else None
         self.sched = Scheduler(self.kv, cfg.max_num_seqs, cfg.max_num_batched_tokens, cfg.max_model_len,
                                mixed_batches=cfg.mixed_batches,
                                reserve_seqs=min(cfg.interactive_reserve_seqs, cfg.max_num_seqs // 4),
@@ -390,7 +400,83 @@ class LLMEngine:
             seq.num_computed = min(seq.num_computed, a)
             del seq.block_hashes[a // bs:]
 
+    # ------------------------------------------------------------------ given-token steps
+    def feed(self, entries, end=()) -> np.ndarray | None:
+        """One engine step over GIVEN tokens, nothing sampled: ``entries`` is [(req_id, tokens, want)] -- the
+        next tokens of each request (admitted at its first entry; it may sit out steps) and the places among them
+        whose logits are wanted.  All entries run as one batch through the same packed upload, cache manager,
+        model step and kernels as scheduled steps: multi-token entries as prompt chunks, single next tokens on
+        the decode path (Scheduler.admit_plan).  ``end``: requests finished after this step -- their blocks and
+        slot go back to the pools.  Returns fp32 logits [wanted, vocab] in entry / want order (None if nothing
+        is wanted)."""
+        try:
+            with self._on_stream(), WS.owned_by(self._ws), (gpu_shared() if self.on_gpu else contextlib.nullcontext()):
+                out = self._feed(entries) if entries else None
+        finally:
+            for rid in end:
+                seq = self._seqs.pop(rid, None)
+                if seq is not None:
+                    self.sched.finish(seq)
+        return out
+
+    @torch.inference_mode()
+    def _feed(self, entries) -> np.ndarray | None:
+        plan = []
+        for rid, toks, _ in entries:
+            seq = self._seqs.get(rid)
+            if seq is None:
+                seq = self._seqs[rid] = Sequence(rid, [], SamplingParams(max_tokens=1 << 30, ignore_eos=True))
+            if seq.output_ids or seq.num_computed != len(seq.prompt_ids):
+                raise RuntimeError(f"{rid} is not a given-token request")
+            plan.append((seq, len(toks)))
+        kind, items, order = self.sched.admit_plan(plan)
+        for (seq, _), (_, toks, _) in zip(plan, entries):
+            seq.prompt_ids.extend(int(t) for t in toks)
+        base = np.concatenate([[0], np.cumsum([b - a for _, a, b in items])])
+        rows = np.asarray([base[order[i]] + int(w) for i, (_, toks, want) in enumerate(entries) for w in want],
+                          dtype=np.int32)
+        for (_, toks, want) in entries:
+            if any(not 0 <= int(w) < len(toks) for w in want):
+                raise ValueError("a wanted place lies outside its entry's tokens")
+        self.stats["steps"] += 1
+        none = np.zeros(0, dtype=np.int32)
+        if kind == "prefill":
+            hidden, d_rows, _, _ = self._prefill_hidden(items, rows, none)
+        elif kind == "mixed":
+            n_pref = next(i for i, (s, a, b) in enumerate(items) if b - a == 1 and a > 0)
+            hidden, d_rows, _, _ = self._mixed_hidden(items[:n_pref], [s for s, _, _ in items[n_pref:]], rows, none)
+        else:
+            seqs = [s for s, _, _ in items]
+            n = len(seqs)
+            max_ctx = max(s.total_len for s in seqs)
+            nsplit, split_len = _decode_plan(self.model, n, max_ctx, self.cfg.max_model_len, graph=False)
+            width = max(len(s.blocks) for s in seqs)
+            ctrl = self._decode_inputs(seqs, n, width, 1)
+            dev = self._to_dev(np.concatenate([ctrl, rows]))
+            v = self._views(dev, n, width, 1)
+            hidden = self._decode_hidden(v, n, nsplit, split_len, 0, v["ids"])
+            d_rows = dev[ctrl.size:]
+        for s, a, b in items:
+            s.num_computed = b
+        n_dec = sum(1 for _, a, b in items if b - a == 1 and a > 0)
+        self.stats["decode_tokens"] += n_dec
+        self.stats["prefill_tokens"] += int(base[-1]) - n_dec
+        if not len(rows):
+            if self.on_gpu:
+                self._read_host(hidden[:1, :1].to(torch.float32).view(torch.int32))  # the step is done when feed returns
+            return None
+        logits = self.model.compute_logits(hidden.index_select(0, d_rows))[:, : self.model.cfg.vocab_size]
+        logits = logits.float().contiguous()
+        if not self.on_gpu:
+            return logits.numpy()
+        return self._read_host(logits.view(torch.int32)).view(np.float32).reshape(logits.shape)
+
     # ------------------------------------------------------------------ helpers
+    def _forward(self, ids, pos, meta: AttnMetadata) -> torch.Tensor:
+        if self.has_state:
+            return self.model.forward(ids, pos, meta, self.kv_caches, state=self.state)
+        return self.model.forward(ids, pos, meta, self.kv_caches)
+
     def _slots_of(self, seq: Sequence, start: int, end: int) -> np.ndarray:
         bs = self.cfg.block_size
         pos = np.arange(start, end)
@@ -435,40 +521,15 @@ class LLMEngine:
         if 0 < n_pref < len(items):
             return self._run_mixed(items[:n_pref], [s for s, _, _ in items[n_pref:]])
         t0 = time.perf_counter()
-        seqs = [s for s, _, _ in items]
-        ids, pos, slots, q_start, ctx = [], [], [], [0], []
-        for s, a, b in items:
-            ids.append(np.asarray(s.all_ids[a:b], dtype=np.int32))
-            pos.append(np.arange(a, b, dtype=np.int32))
-            slots.append(self._slots_of(s, a, b))
-            q_start.append(q_start[-1] + (b - a))
-            ctx.append(b)
         # rows to sample: the last token of every chunk that completes its prompt.  Uploaded with the step's
         # inputs: a separate pageable upload after the forward is a synchronous copy queued behind it, which
         # held the host until the forward finished and left the GPU idle while the LM head and sampler launched
         samp = [i for i, (s, a, b) in enumerate(items) if b == s.total_len]
-        width = max(len(s.blocks) for s in seqs)
-        packed = np.concatenate([np.concatenate(ids), np.concatenate(pos), np.concatenate(slots),
-                                 np.asarray(q_start, dtype=np.int32), np.asarray(ctx, dtype=np.int32),
-                                 self._block_table(seqs, width).reshape(-1),
-                                 np.asarray([q_start[i + 1] - 1 for i in samp], dtype=np.int32),
-                                 np.asarray([items[i][0].slot for i in samp], dtype=np.int32)])
-        dev = self._to_dev(packed)
-        th = time.perf_counter()
-        self.stats["host_prefill_prep_s"] += th - t0
-        T, n = q_start[-1], len(seqs)
-        o = 0
-        d_ids = dev[o:o + T]; o += T
-        d_pos = dev[o:o + T]; o += T
-        d_slot = dev[o:o + T]; o += T
-        d_qs = dev[o:o + n + 1]; o += n + 1
-        d_ctx = dev[o:o + n]; o += n
-        d_bt = dev[o:o + n * width].view(n, width); o += n * width
-        d_rows = dev[o:o + len(samp)]; o += len(samp)
-        d_samp_slots = dev[o:o + len(samp)]
-        meta = AttnMetadata(q_start=d_qs, ctx_len=d_ctx, block_tables=d_bt, slot_mapping=d_slot,
-                            max_q_len=max(b - a for _, a, b in items), num_seqs=n, num_tokens=T)
-        hidden = self.model.forward(d_ids, d_pos, meta, self.kv_caches)
+        ends = np.cumsum([b - a for _, a, b in items])
+        hidden, d_rows, d_samp_slots, th = self._prefill_hidden(
+            items, np.asarray([ends[i] - 1 for i in samp], dtype=np.int32),
+            np.asarray([items[i][0].slot for i in samp], dtype=np.int32), t0)
+        T = int(ends[-1])
         tp = self.model.tp
         if samp:  # LM head + sampler queued right behind the forward
             toks_d = self._sample(hidden.index_select(0, d_rows), d_samp_slots)
@@ -493,6 +554,45 @@ class LLMEngine:
         self.stats["prefill_s"] += time.perf_counter() - t0
         return finished
 
+    def _prefill_hidden(self, items, rows: np.ndarray, row_slots: np.ndarray, t0: float | None = None):
+        """Upload one step of prompt chunks ``items`` [(seq, start, end)] and launch the model over them.
+        ``rows``: token rows of the step whose hidden state the caller reads next (sampling rows), ``row_slots``:
+        their sampler slots -- both go up in the step's one packed buffer.  Returns (hidden [T, H], rows on
+        device, row_slots on device, time the launch began)."""
+        t0 = time.perf_counter() if t0 is None else t0
+        seqs = [s for s, _, _ in items]
+        ids, pos, slots, q_start, ctx = [], [], [], [0], []
+        for s, a, b in items:
+            ids.append(np.asarray(s.all_ids[a:b], dtype=np.int32))
+            pos.append(np.arange(a, b, dtype=np.int32))
+            slots.append(self._slots_of(s, a, b))
+            q_start.append(q_start[-1] + (b - a))
+            ctx.append(b)
+        width = max(len(s.blocks) for s in seqs)
+        packed = np.concatenate([np.concatenate(ids), np.concatenate(pos), np.concatenate(slots),
+                                 np.asarray(q_start, dtype=np.int32), np.asarray(ctx, dtype=np.int32),
+                                 self._block_table(seqs, width).reshape(-1),
+                                 np.asarray(rows, dtype=np.int32), np.asarray(row_slots, dtype=np.int32),
+                                 np.asarray([s.slot for s in seqs], dtype=np.int32)])
+        dev = self._to_dev(packed)
+        th = time.perf_counter()
+        self.stats["host_prefill_prep_s"] += th - t0
+        T, n = q_start[-1], len(seqs)
+        o = 0
+        d_ids = dev[o:o + T]; o += T
+        d_pos = dev[o:o + T]; o += T
+        d_slot = dev[o:o + T]; o += T
+        d_qs = dev[o:o + n + 1]; o += n + 1
+        d_ctx = dev[o:o + n]; o += n
+        d_bt = dev[o:o + n * width].view(n, width); o += n * width
+        d_rows = dev[o:o + len(rows)]; o += len(rows)
+        d_row_slots = dev[o:o + len(row_slots)]; o += len(row_slots)
+        d_state = dev[o:o + n]
+        meta = AttnMetadata(q_start=d_qs, ctx_len=d_ctx, block_tables=d_bt, slot_mapping=d_slot,
+                            max_q_len=max(b - a for _, a, b in items), num_seqs=n, num_tokens=T,
+                            state_slots=d_state)
+        return self._forward(d_ids, d_pos, meta), d_rows, d_row_slots, th
+
     def _run_mixed(self, pitems, dseqs) -> list[Sequence]:
         """One step of prefill chunks plus one decode token for every decode-ready sequence (stall-free
         batching): the decode rows ride in the prefill step's GEMMs (M = prefill tokens + decode rows,
@@ -500,66 +600,16 @@ class LLMEngine:
         their attention runs on the split-KV decode kernel.  Inputs go up as one packed int32 buffer: the
         prefill part built per chunk, the decode part from the per-slot block table (_decode_inputs)."""
         t0 = time.perf_counter()
-        bs = self.cfg.block_size
-        n_pref, n_dec = len(pitems), len(dseqs)
-        ids, pos, slots, q_start, ctx = [], [], [], [0], []
-        for s, a, b in pitems:
-            ids.append(np.asarray(s.all_ids[a:b], dtype=np.int32))
-            pos.append(np.arange(a, b, dtype=np.int32))
-            slots.append(self._slots_of(s, a, b))
-            q_start.append(q_start[-1] + (b - a))
-            ctx.append(b)
-        Tp = q_start[-1]
-        T = Tp + n_dec
+        n_dec = len(dseqs)
         pseqs = [s for s, _, _ in pitems]
-        wp = max(len(s.blocks) for s in pseqs)
-        max_ctx = max(s.total_len for s in dseqs)
-        wd = -(-max_ctx // bs)
-        dec = self._decode_inputs(dseqs, n_dec, wd, 1)
-        lay = _ctrl_layout(n_dec, wd, 1)
-
-        def part(name):
-            o, shape = lay[name]
-            return dec[o:o + int(np.prod(shape))]
-
-        d_ids, d_pos, d_slot, d_ctx, d_samp, d_bt = (part(k) for k in ("ids", "pos", "slot", "ctx", "slots", "bt"))
+        ends = np.cumsum([b - a for _, a, b in pitems])
+        Tp = int(ends[-1])
         # rows to sample: the last token of every prefill chunk that completes its prompt, then every decode row
         done = [i for i, (s, a, b) in enumerate(pitems) if b == s.total_len]
-        samp_rows = np.concatenate([np.asarray([q_start[i + 1] - 1 for i in done], dtype=np.int32),
-                                    np.arange(Tp, T, dtype=np.int32)])
-        samp_slots = np.concatenate([np.asarray([pseqs[i].slot for i in done], dtype=np.int32), d_samp])
-        packed = np.concatenate([
-            *ids, d_ids, *pos, d_pos, *slots, d_slot,                       # [T] x 3
-            np.asarray(q_start, dtype=np.int32), np.asarray(ctx, dtype=np.int32),
-            self._block_table(pseqs, wp).reshape(-1),                       # prefill chunks
-            np.arange(n_dec + 1, dtype=np.int32), d_ctx, d_bt,              # decode rows
-            samp_rows, samp_slots])
-        dev = self._to_dev(packed)
-        th = time.perf_counter()
-        self.stats["host_prefill_prep_s"] += th - t0
-        o = 0
-        t_ids = dev[o:o + T]; o += T
-        t_pos = dev[o:o + T]; o += T
-        t_slot = dev[o:o + T]; o += T
-        p_qs = dev[o:o + n_pref + 1]; o += n_pref + 1
-        p_ctx = dev[o:o + n_pref]; o += n_pref
-        p_bt = dev[o:o + n_pref * wp].view(n_pref, wp); o += n_pref * wp
-        q_qs = dev[o:o + n_dec + 1]; o += n_dec + 1
-        q_ctx = dev[o:o + n_dec]; o += n_dec
-        q_bt = dev[o:o + n_dec * wd].view(n_dec, wd); o += n_dec * wd
-        ns = len(samp_rows)
-        t_rows = dev[o:o + ns]; o += ns
-        t_samp = dev[o:o + ns]
-        nsplit, split_len = _decode_plan(self.model, n_dec, max_ctx, self.cfg.max_model_len, graph=False)
-        hq, dh = self.model.hq, self.model.head_dim
-        meta = AttnMetadata(q_start=p_qs, ctx_len=p_ctx, block_tables=p_bt, slot_mapping=t_slot,
-                            max_q_len=max(b - a for _, a, b in pitems), num_seqs=n_pref, num_tokens=Tp)
-        meta.extra["decode_rows"] = (Tp, AttnMetadata(
-            q_start=q_qs, ctx_len=q_ctx, block_tables=q_bt, slot_mapping=t_slot[Tp:], max_q_len=1, num_seqs=n_dec,
-            num_tokens=n_dec, is_decode=True, num_splits=nsplit, split_len=split_len,
-            part_o=self._part_o[: nsplit * n_dec * hq * dh] if self.on_gpu else None,
-            part_ml=self._part_ml[: nsplit * n_dec * hq * 2] if self.on_gpu else None))
-        hidden = self.model.forward(t_ids, t_pos, meta, self.kv_caches)
+        samp_rows = np.concatenate([np.asarray([ends[i] - 1 for i in done], dtype=np.int32),
+                                    np.arange(Tp, Tp + n_dec, dtype=np.int32)])
+        hidden, t_rows, t_samp, th = self._mixed_hidden(pitems, dseqs, samp_rows,
+                                                        np.asarray([pseqs[i].slot for i in done], dtype=np.int32), t0)
         toks_d = self._sample(hidden.index_select(0, t_rows), t_samp)
         t1 = time.perf_counter()
         self.stats["host_prefill_launch_s"] += t1 - th
@@ -591,6 +641,74 @@ class LLMEngine:
         self.stats["mixed_steps"] += 1
         self.stats["prefill_s"] += time.perf_counter() - t0
         return finished
+
+    def _mixed_hidden(self, pitems, dseqs, rows: np.ndarray, prefill_row_slots: np.ndarray, t0: float | None = None):
+        """Upload and launch one mixed step: prompt chunks ``pitems`` (token rows [0, Tp)) and one token of each
+        sequence of ``dseqs`` (rows [Tp, Tp + len(dseqs)), attended by the decode kernels).  ``rows``: token rows
+        the caller reads next; ``prefill_row_slots``: sampler slots of the prefill rows among them (the decode
+        rows' slots follow from ``dseqs``).  Returns (hidden [T, H], rows on device, their sampler slots on
+        device, time the launch began)."""
+        t0 = time.perf_counter() if t0 is None else t0
+        bs = self.cfg.block_size
+        n_pref, n_dec = len(pitems), len(dseqs)
+        ids, pos, slots, q_start, ctx = [], [], [], [0], []
+        for s, a, b in pitems:
+            ids.append(np.asarray(s.all_ids[a:b], dtype=np.int32))
+            pos.append(np.arange(a, b, dtype=np.int32))
+            slots.append(self._slots_of(s, a, b))
+            q_start.append(q_start[-1] + (b - a))
+            ctx.append(b)
+        Tp = q_start[-1]
+        T = Tp + n_dec
+        pseqs = [s for s, _, _ in pitems]
+        wp = max(len(s.blocks) for s in pseqs)
+        max_ctx = max(s.total_len for s in dseqs)
+        wd = -(-max_ctx // bs)
+        dec = self._decode_inputs(dseqs, n_dec, wd, 1)
+        lay = _ctrl_layout(n_dec, wd, 1)
+
+        def part(name):
+            o, shape = lay[name]
+            return dec[o:o + int(np.prod(shape))]
+
+        d_ids, d_pos, d_slot, d_ctx, d_samp, d_bt = (part(k) for k in ("ids", "pos", "slot", "ctx", "slots", "bt"))
+        samp_slots = np.concatenate([np.asarray(prefill_row_slots, dtype=np.int32), d_samp])[: len(rows)]
+        packed = np.concatenate([
+            *ids, d_ids, *pos, d_pos, *slots, d_slot,                       # [T] x 3
+            np.asarray(q_start, dtype=np.int32), np.asarray(ctx, dtype=np.int32),
+            self._block_table(pseqs, wp).reshape(-1),                       # prefill chunks
+            np.arange(n_dec + 1, dtype=np.int32), d_ctx, d_bt,              # decode rows
+            np.asarray(rows, dtype=np.int32), samp_slots,
+            np.asarray([s.slot for s in pseqs], dtype=np.int32), d_samp])   # state slots
+        dev = self._to_dev(packed)
+        th = time.perf_counter()
+        self.stats["host_prefill_prep_s"] += th - t0
+        o = 0
+        t_ids = dev[o:o + T]; o += T
+        t_pos = dev[o:o + T]; o += T
+        t_slot = dev[o:o + T]; o += T
+        p_qs = dev[o:o + n_pref + 1]; o += n_pref + 1
+        p_ctx = dev[o:o + n_pref]; o += n_pref
+        p_bt = dev[o:o + n_pref * wp].view(n_pref, wp); o += n_pref * wp
+        q_qs = dev[o:o + n_dec + 1]; o += n_dec + 1
+        q_ctx = dev[o:o + n_dec]; o += n_dec
+        q_bt = dev[o:o + n_dec * wd].view(n_dec, wd); o += n_dec * wd
+        ns = len(rows)
+        t_rows = dev[o:o + ns]; o += ns
+        t_samp = dev[o:o + len(samp_slots)]; o += len(samp_slots)
+        p_state = dev[o:o + n_pref]; o += n_pref
+        q_state = dev[o:o + n_dec]
+        nsplit, split_len = _decode_plan(self.model, n_dec, max_ctx, self.cfg.max_model_len, graph=False)
+        hq, dh = self.model.hq, self.model.head_dim
+        meta = AttnMetadata(q_start=p_qs, ctx_len=p_ctx, block_tables=p_bt, slot_mapping=t_slot,
+                            max_q_len=max(b - a for _, a, b in pitems), num_seqs=n_pref, num_tokens=Tp,
+                            state_slots=p_state)
+        meta.extra["decode_rows"] = (Tp, AttnMetadata(
+            q_start=q_qs, ctx_len=q_ctx, block_tables=q_bt, slot_mapping=t_slot[Tp:], max_q_len=1, num_seqs=n_dec,
+            num_tokens=n_dec, is_decode=True, num_splits=nsplit, split_len=split_len,
+            part_o=self._part_o[: nsplit * n_dec * hq * dh] if self.on_gpu else None,
+            part_ml=self._part_ml[: nsplit * n_dec * hq * 2] if self.on_gpu else None, state_slots=q_state))
+        return self._forward(t_ids, t_pos, meta), t_rows, t_samp, th
 
     # ------------------------------------------------------------------ decode
     @staticmethod
@@ -710,12 +828,19 @@ class LLMEngine:
                           pre_ml=self._pre_ml[: npl * B * hq * 2] if self.on_gpu else None, rg=CASCADE_RG)
         for j in range(K):
             ids = v["ids"] if j == 0 else out_tokens[j - 1]
-            meta = AttnMetadata(q_start=v["qs"], ctx_len=v["ctx"][j], block_tables=v["bt"], slot_mapping=v["slot"][j],
-                                max_q_len=1, num_seqs=B, num_tokens=B, is_decode=True, num_splits=nsplit,
-                                split_len=split_len, part_o=part_o, part_ml=part_ml, cascade=cas)
-            hidden = self.model.forward(ids, v["pos"][j], meta, self.kv_caches)
+            hidden = self._decode_hidden(v, B, nsplit, split_len, j, ids, part_o, part_ml, cas)
             self._sample(hidden, v["slots"], out=out_tokens[j])
         return out_tokens
+
+    def _decode_hidden(self, v, B, nsplit, split_len, j, ids, part_o=None, part_ml=None, cas=None) -> torch.Tensor:
+        """The model over step ``j`` of a decode window's control views ``v`` (one token per row)."""
+        if part_o is None and self.on_gpu:
+            hq, d = self.model.hq, self.model.head_dim
+            part_o, part_ml = self._part_o[: nsplit * B * hq * d], self._part_ml[: nsplit * B * hq * 2]
+        meta = AttnMetadata(q_start=v["qs"], ctx_len=v["ctx"][j], block_tables=v["bt"], slot_mapping=v["slot"][j],
+                            max_q_len=1, num_seqs=B, num_tokens=B, is_decode=True, num_splits=nsplit,
+                            split_len=split_len, part_o=part_o, part_ml=part_ml, cascade=cas, state_slots=v["slots"])
+        return self._forward(ids, v["pos"][j], meta)
 
     def _sample(self, hidden: torch.Tensor, slots: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
         """LM head + sampler.  Under TP the vocab-parallel sampler runs on this rank's logit shard
@@ -1024,6 +1149,8 @@ class LLMEngine:
 
     def _detok_all(self, ids) -> str:
         """The text IncrementalDetokenizer would have produced for ``ids`` (same bytes, same decoder)."""
+        if self.tok is None:  # token-id clients (no tokenizer attached): no text
+            return ""
         tb = getattr(self.tok, "token_bytes", None)
         if tb is None:
             return "".join(self.tok.decode([t]) for t in ids)

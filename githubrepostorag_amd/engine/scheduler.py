@@ -235,6 +235,39 @@ class Scheduler:
                     out.append(s)
         return out
 
+    def admit_plan(self, plan):
+        """A step whose contents the caller fixes (replaying a recorded schedule, teacher-forced scoring):
+        ``plan`` is [(seq, n)] -- the next n tokens of each sequence, all in one batch.  A sequence not yet
+        running is admitted here (a sequence slot); every sequence gets the KV blocks its tokens need from the
+        same pool and allocator as scheduled steps.  Raises when the slots or the pool do not hold the plan
+        (nothing is preempted: the caller owns the schedule).  Returns (kind, items, order): items as
+        schedule() returns them -- chunks first, then the one-token rows of sequences already past their first
+        token, which take the decode kernels -- and order[i] = the index in items of plan entry i."""
+        with self.lock:
+            chunks, rows = [], []
+            for i, (seq, n) in enumerate(plan):
+                if n <= 0:
+                    raise ValueError("a plan entry needs at least one token")
+                if seq.status != SeqStatus.RUNNING:
+                    if not self.free_slots or len(self.running) >= self.max_num_seqs:
+                        raise RuntimeError(f"no free sequence slot for {seq.req_id} ({self.max_num_seqs} live)")
+                    seq.slot = self.free_slots.pop()
+                    seq.status = SeqStatus.RUNNING
+                    self.running.append(seq)
+                a = seq.num_computed
+                if a + n > self.max_model_len:
+                    raise ValueError(f"{seq.req_id}: {a + n} tokens exceed max_model_len {self.max_model_len}")
+                if not self.kv.ensure(seq, a + n):
+                    raise MemoryError(f"KV pool exhausted admitting {n} tokens of {seq.req_id} "
+                                      f"({self.kv.num_free} blocks free)")
+                (rows if n == 1 and a > 0 else chunks).append((i, (seq, a, a + n)))
+            both = chunks + rows
+            order = [0] * len(both)
+            for k, (i, _) in enumerate(both):
+                order[i] = k
+            kind = "mixed" if chunks and rows else "prefill" if chunks else "decode"
+            return kind, [it for _, it in both], order
+
     @staticmethod
     def prefill_target(seq: Sequence) -> int:
         return seq.total_len - (1 if seq.output_ids else 0)

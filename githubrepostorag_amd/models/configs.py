@@ -7,7 +7,9 @@ unless a local HF-format directory is given (see models/weights.py).
 """
 from __future__ import annotations
 
-from dataclasses import asdict, dataclass, replace
+import json
+from dataclasses import asdict, dataclass, field, replace
+from pathlib import Path
 
 
 @dataclass(frozen=True)
@@ -68,6 +70,207 @@ class EncoderConfig:
 
     def to_dict(self):
         return asdict(self)
+
+
+# ---------------------------------------------------------------------------------------------- hybrid decoders
+# Decoders whose layer list is data: every layer names its sequence mixer ("parallel": softmax attention with a
+# sink beside decay linear attention; "mingru": a gated recurrence) and its feed-forward, and a span of layers
+# may be run several times in a row with shared weights (a loop), every pass with its own cache and state.
+
+
+@dataclass(frozen=True)
+class SinkAttnSpec:
+    """Softmax attention with a per-head sink, GQA, partial rotary and RMS-normed values."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    rot_dims: int
+    rot_base: float
+
+
+@dataclass(frozen=True)
+class DecayAttnSpec:
+    """Linear attention with a fixed decay per head and a [dim, vdim] state per head."""
+    heads: int
+    dim: int
+    vdim: int
+    decay: tuple
+
+
+@dataclass(frozen=True)
+class MixerSpec:
+    kind: str  # "parallel" | "mingru"
+    left: SinkAttnSpec | None = None
+    right: DecayAttnSpec | None = None
+    left_scale: float = 1.0
+    right_scale: float = 1.0
+    width: int = 0  # mingru state width
+
+
+@dataclass(frozen=True)
+class GLUSpec:
+    kind: str  # "dense"
+    ff: int
+    limit: float
+
+
+@dataclass(frozen=True)
+class HybridLayerSpec:
+    mixer: MixerSpec
+    mlp: GLUSpec | None
+
+
+@dataclass(frozen=True)
+class HybridConfig:
+    name: str
+    vocab_size: int
+    hidden_size: int
+    norm_eps: float
+    layers: tuple
+    loop_start: int = 0
+    loop_stop: int = 0
+    loop_times: int = 1
+    arch: str = "zofesun"
+    max_position: int = 1 << 20  # the design has no position limit of its own: the engine's max_model_len bounds it
+    tie_word_embeddings: bool = False
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    def layer_runs(self) -> list:
+        """[(layer index, pass number, first of its pass)] in execution order: layers before the loop once,
+        the looped span ``loop_times`` times, the rest once.  Every run has its own cache / state."""
+        a, b, n = self.loop_start, self.loop_stop, len(self.layers)
+        if not (0 <= a <= b <= n) or self.loop_times < 1:
+            raise ValueError(f"loop [{a}, {b}) x {self.loop_times} does not fit {n} layers")
+        runs = [(i, 0, False) for i in range(a)]
+        for t in range(self.loop_times if b > a else 0):
+            runs += [(i, t, i == a) for i in range(a, b)]
+        runs += [(i, 0, False) for i in range(b, n)]
+        return runs
+
+    def to_dict(self):
+        return asdict(self)
+
+    def param_count(self) -> int:
+        H = self.hidden_size
+        n = 2 * self.vocab_size * H + 2 * H + 1 + self.loop_times * H
+        for L in self.layers:
+            n += 4 * (2 * H + 1)
+            m = L.mixer
+            if m.kind == "mingru":
+                n += 3 * m.width * H + 2 * m.width + H * m.width
+            else:
+                l, r = m.left, m.right
+                n += H * (l.heads * l.dim + l.kv_heads * (l.dim + l.vdim)) + l.heads + l.heads * l.vdim * H
+                n += H * r.heads * (2 * r.dim + 2 * r.vdim) + r.heads * r.vdim * (H + 1)
+            if L.mlp is not None:
+                n += 3 * H * L.mlp.ff
+        return n
+
+
+def hybrid_config_from_dict(d: dict, name: str = "zofesun") -> HybridConfig:
+    """The design's config.json: sizes and constants are all read from it."""
+    layers = []
+    for e in d["layers"]:
+        kind, m = e["type"], e["mixer"]
+        if kind == "parallel":
+            l, r = m["left"], m["right"]
+            left = SinkAttnSpec(int(l["heads"]), int(l["kv_heads"]), int(l["dim"]), int(l["vdim"]), float(l["scale"]),
+                                int(l["rot"]["dims"]), float(l["rot"]["base"]))
+            right = DecayAttnSpec(int(r["heads"]), int(r["dim"]), int(r["vdim"]), tuple(float(x) for x in r["decay"]))
+            if left.heads % left.kv_heads or left.rot_dims % 2 or left.rot_dims > left.dim:
+                raise ValueError(f"bad attention sizes {l}")
+            if len(right.decay) != right.heads:
+                raise ValueError("one decay per linear-attention head")
+            mixer = MixerSpec("parallel", left, right, float(m["left_scale"]), float(m["right_scale"]))
+        elif kind == "mingru":
+            mixer = MixerSpec("mingru", width=int(m["width"]))
+        else:
+            raise ValueError(f"unknown mixer type {kind!r}")
+        f = e.get("mlp")
+        if f is None:
+            mlp = None
+        elif f.get("kind", "dense") == "dense":
+            mlp = GLUSpec("dense", int(f["ff"]), float(f["limit"]))
+        else:
+            raise ValueError(f"unknown feed-forward kind {f.get('kind')!r}")
+        layers.append(HybridLayerSpec(mixer, mlp))
+    loop = d.get("loop") or {}
+    return HybridConfig(name, int(d["vocab"]), int(d["width"]), float(d["norm"]["eps"]), tuple(layers),
+                        int(loop.get("start", 0)), int(loop.get("stop", 0)), int(loop.get("times", 1)))
+
+
+def hybrid_config_to_dict(cfg: HybridConfig) -> dict:
+    """Back to the config.json form (checkpoint export, tests)."""
+    layers = []
+    for L in cfg.layers:
+        m = L.mixer
+        if m.kind == "mingru":
+            mixer = {"width": m.width}
+        else:
+            l, r = m.left, m.right
+            mixer = {"left": {"heads": l.heads, "kv_heads": l.kv_heads, "dim": l.dim, "vdim": l.vdim, "scale": l.scale,
+                              "rot": {"dims": l.rot_dims, "base": l.rot_base}},
+                     "left_scale": m.left_scale,
+                     "right": {"heads": r.heads, "dim": r.dim, "vdim": r.vdim, "decay": list(r.decay)},
+                     "right_scale": m.right_scale}
+        mlp = None if L.mlp is None else {"kind": L.mlp.kind, "ff": L.mlp.ff, "limit": L.mlp.limit}
+        layers.append({"type": m.kind, "mixer": mixer, "mlp": mlp})
+    return {"architecture": "Zofesun", "vocab": cfg.vocab_size, "width": cfg.hidden_size,
+            "norm": {"eps": cfg.norm_eps}, "layers": layers,
+            "loop": {"start": cfg.loop_start, "stop": cfg.loop_stop, "times": cfg.loop_times}}
+
+
+def zofesun_config(name: str, vocab: int, width: int, n_layers: int, *, heads: int, kv_heads: int, dim: int,
+                   vdim: int, lin_heads: int, lin_dim: int, lin_vdim: int, ff: int, mingru_every: int = 0,
+                   rot_dims: int | None = None, rot_base: float = 10000.0, loop=(0, 0, 1), limit: float = 7.0,
+                   eps: float = 1e-5) -> HybridConfig:
+    """A regular Zofesun stack for benches and plumbing tests: ``n_layers`` parallel layers, every
+    ``mingru_every``-th one (if any) a minGRU layer instead, decays spread over the linear heads."""
+    left = SinkAttnSpec(heads, kv_heads, dim, vdim, dim ** -0.5, dim if rot_dims is None else rot_dims, rot_base)
+    decay = tuple(1.0 - 2.0 ** (-2.0 - 6.0 * i / max(1, lin_heads - 1)) for i in range(lin_heads))
+    right = DecayAttnSpec(lin_heads, lin_dim, lin_vdim, decay)
+    par = HybridLayerSpec(MixerSpec("parallel", left, right, 0.7, 0.9), GLUSpec("dense", ff, limit))
+    gru = HybridLayerSpec(MixerSpec("mingru", width=width), GLUSpec("dense", ff, limit))
+    layers = tuple(gru if mingru_every and (i + 1) % mingru_every == 0 else par for i in range(n_layers))
+    return HybridConfig(name, vocab, width, eps, layers, *loop)
+
+
+HYBRIDS = {
+    # plumbing-test sizes (CPU tier) and two bench sizes shaped like the layers of a 1.5B / 7B decoder
+    "zofesun-tiny": zofesun_config("zofesun-tiny", 384, 128, 3, heads=4, kv_heads=2, dim=48, vdim=16, lin_heads=2,
+                                   lin_dim=16, lin_vdim=24, ff=192, mingru_every=2, rot_dims=16, loop=(1, 3, 2)),
+    "zofesun-1b": zofesun_config("zofesun-1b", 32768, 1536, 8, heads=12, kv_heads=2, dim=128, vdim=128,
+                                 lin_heads=12, lin_dim=128, lin_vdim=128, ff=8960, mingru_every=4),
+    "zofesun-7b": zofesun_config("zofesun-7b", 32768, 3584, 4, heads=28, kv_heads=4, dim=128, vdim=128,
+                                 lin_heads=28, lin_dim=128, lin_vdim=128, ff=18944, mingru_every=4),
+}
+
+
+def config_from_dir(path) -> DecoderConfig | HybridConfig:
+    """The decoder config a checkpoint directory's config.json describes: the hybrid design by its
+    ``architecture`` key, the HF families by ``model_type``."""
+    d = json.loads((Path(path) / "config.json").read_text())
+    arch = str(d.get("architecture", "")).lower()
+    if arch == "zofesun":
+        return hybrid_config_from_dict(d, Path(path).name or "zofesun")
+    mt = str(d.get("model_type", "")).lower()
+    if mt == "gpt2":
+        return DecoderConfig(Path(path).name, d["vocab_size"], d["n_embd"], d.get("n_inner") or 4 * d["n_embd"],
+                             d["n_layer"], d["n_head"], d["n_head"], d["n_embd"] // d["n_head"],
+                             d.get("layer_norm_epsilon", 1e-5), 0.0, d.get("n_positions", 1024), True, True, "gpt2")
+    if mt.startswith("qwen2"):
+        hd = d.get("head_dim") or d["hidden_size"] // d["num_attention_heads"]
+        return DecoderConfig(Path(path).name, d["vocab_size"], d["hidden_size"], d["intermediate_size"],
+                             d["num_hidden_layers"], d["num_attention_heads"],
+                             d.get("num_key_value_heads", d["num_attention_heads"]), hd, d.get("rms_norm_eps", 1e-6),
+                             d.get("rope_theta", 1e6), d.get("max_position_embeddings", 32768),
+                             d.get("tie_word_embeddings", False))
+    raise ValueError(f"config.json of {path} names no architecture this engine serves")
 
 
 DECODERS = {
@@ -138,8 +341,9 @@ def _key(name: str) -> str:
     return ALIASES.get(k, k.split("/")[-1])
 
 
-def decoder_config(name: str, **overrides) -> DecoderConfig:
-    cfg = DECODERS[_key(name)]
+def decoder_config(name: str, **overrides):
+    k = _key(name)
+    cfg = HYBRIDS[k] if k in HYBRIDS else DECODERS[k]
     return replace(cfg, **overrides) if overrides else cfg
 
 

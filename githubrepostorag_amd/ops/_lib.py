@@ -79,6 +79,15 @@ _SIGS = {
     "grag_gemm_w4": [P, P, P, P, P, I, I, I, I, I, I, I, I, I, I, P, P],
     "grag_gemm_w4_has": [I, I],
     "grag_err_alloc": [P],
+    "grag_embed_f32": [P, P, P, I, I, I, I, P],
+    "grag_dyt_residual": [P, F, P, P, P, P, P, F, P, P, P, I, I, I, P],
+    "grag_rope_vnorm_store": [P, I, I, I, I, P, P, I, P, P, P, P, I, I, I, I, I, I, I, ctypes.c_long, F, I, P],
+    "grag_sink_attn_prefill": [P, P, P, P, I, P, I, P, P, P, I, I, I, I, I, I, I, F, F, I, I, P],
+    "grag_sink_attn_decode": [P, P, P, P, I, P, I, P, P, I, I, I, I, I, I, F, F, I, I, P],
+    "grag_decay_attn_scan": [P, I, I, I, I, P, P, P, P, P, P, I, I, I, I, I, I, P],
+    "grag_gated_rmsnorm": [P, P, P, I, I, P, I, I, I, F, F, I, P],
+    "grag_mingru_scan": [P, I, I, I, I, P, P, P, P, P, P, P, I, I, I, I, P],
+    "grag_clamped_glu": [P, P, I, I, F, F, I, P],
     "grag_attn_decode_xcd": [I],
 }
 
@@ -146,7 +155,7 @@ def call(name: str, *args) -> None:
 
 
 # ---------------------------------------------------------------- device index guard (csrc/kernels/common.h)
-ERR_UNITS = ("norm", "elementwise", "attention", "gemm_tile", "gemm_stream")
+ERR_UNITS = ("norm", "elementwise", "attention", "gemm_tile", "gemm_stream", "seqmix")
 ERR_CODES = {1 << 0: "embed_gather: token id >= vocab", 1 << 1: "qkv_rope_kvstore: KV slot id >= cache slots",
              1 << 2: "qkv_rope_kvstore: position >= RoPE table rows",
              1 << 3: "prefill attention: block-table entry >= KV blocks",

@@ -123,6 +123,8 @@ class AttnMetadata:
     # shared-prefix decode (prefix_groups / csrc/kernels/attention.hip paged_decode_prefix_kernel): a Cascade or
     # None.  The fp32 reference needs none of it (the same keys, attended in one pass)
     cascade: "Cascade | None" = None
+    # recurrent-state slot of every sequence [nseq] int32 (models with carried state: ops/recurrent.py)
+    state_slots: torch.Tensor | None = None
 
 
 @dataclass
@@ -407,4 +409,66 @@ def varlen_attention(qkv: torch.Tensor, seq_start: torch.Tensor, seq_len: torch.
     call("grag_varlen_attention", base, base + H * D * es, base + 2 * H * D * es, qkv.stride(0), ptr(out),
          out.stride(0), ptr(seq_start), ptr(seq_len), seq_len.numel(), max_len, H, H, D, float(scale),
          1 if causal else 0)
+    return out
+
+
+# ---------------------------------------------------------------------------------------------- sink attention
+def sink_attention_ref(q, k_cache, v_cache, meta: AttnMetadata, scale: float, sinks: torch.Tensor):
+    """fp32: q [T, H, d], k_cache [blocks, G, BS, d], v_cache [blocks, G, BS, vd] -> [T, H, vd].  Causal softmax
+    whose denominator also holds exp(sinks[h]): one more logit with no key and no value."""
+    T, H, d = q.shape
+    G, BS, vd = v_cache.shape[1], v_cache.shape[2], v_cache.shape[3]
+    R = H // G
+    out = torch.zeros(T, H, vd, dtype=torch.float32, device=q.device)
+    qs, cl = meta.q_start.tolist(), meta.ctx_len.tolist()
+    for s in range(meta.num_seqs):
+        a, b = qs[s], qs[s + 1]
+        ql, ctx = b - a, cl[s]
+        if ql <= 0:
+            continue
+        blocks = meta.block_tables[s, : -(-ctx // BS)].long()
+        K = k_cache[blocks].permute(0, 2, 1, 3).reshape(-1, G, d)[:ctx].float().repeat_interleave(R, dim=1)
+        V = v_cache[blocks].permute(0, 2, 1, 3).reshape(-1, G, vd)[:ctx].float().repeat_interleave(R, dim=1)
+        sc = torch.einsum("phd,khd->hpk", q[a:b].float(), K) * scale
+        pos = torch.arange(ctx - ql, ctx, device=q.device)[:, None]
+        sc = sc.masked_fill((torch.arange(ctx, device=q.device)[None, :] > pos)[None], float("-inf"))
+        sk = sinks.float().view(H, 1, 1).expand(H, ql, 1)
+        p = torch.softmax(torch.cat([sc, sk], dim=-1), dim=-1)[..., :ctx]
+        out[a:b] = torch.einsum("hpk,khd->phd", p, V)
+    return out
+
+
+def sink_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, meta: AttnMetadata, scale: float,
+                   sinks: torch.Tensor, out: torch.Tensor | None = None, out_scale: float = 1.0) -> torch.Tensor:
+    """Paged causal attention with a sink term, key size != value size allowed: q [T, H, d] -> out [T, H*vd]
+    (``out`` may be a column slice of a wider buffer), multiplied by ``out_scale``.  Prefill chunks run the
+    tiled kernel, decode rows (one query per sequence) the decode kernel; a mixed step runs both."""
+    T, H, d = q.shape
+    G, BS, vd = v_cache.shape[1], v_cache.shape[2], v_cache.shape[3]
+    if out is None:
+        out = torch.empty(T, H * vd, dtype=q.dtype, device=q.device)
+    dec = meta.extra.get("decode_rows")
+    if dec is not None:
+        Tp, dmeta = dec
+        pmeta = AttnMetadata(q_start=meta.q_start, ctx_len=meta.ctx_len, block_tables=meta.block_tables,
+                             slot_mapping=meta.slot_mapping, max_q_len=meta.max_q_len, num_seqs=meta.num_seqs,
+                             num_tokens=Tp)
+        sink_attention(q[:Tp], k_cache, v_cache, pmeta, scale, sinks, out[:Tp], out_scale)
+        sink_attention(q[Tp:], k_cache, v_cache, dmeta, scale, sinks, out[Tp:], out_scale)
+        return out
+    if T == 0:
+        return out
+    if not q.is_cuda:
+        out.copy_((sink_attention_ref(q, k_cache, v_cache, meta, scale, sinks) * out_scale).reshape(T, H * vd))
+        return out
+    assert q.is_contiguous() and out.stride(1) == 1 and sinks.dtype == torch.float32
+    dt = 0 if q.dtype == torch.bfloat16 else 1
+    if meta.is_decode and meta.max_q_len == 1:
+        call("grag_sink_attn_decode", ptr(q), ptr(k_cache), ptr(v_cache), ptr(out), out.stride(0),
+             ptr(meta.block_tables), meta.block_tables.stride(0), ptr(meta.ctx_len), ptr(sinks), meta.num_seqs, H, G,
+             d, vd, BS, float(scale), float(out_scale), k_cache.shape[0], dt)
+    else:
+        call("grag_sink_attn_prefill", ptr(q), ptr(k_cache), ptr(v_cache), ptr(out), out.stride(0),
+             ptr(meta.block_tables), meta.block_tables.stride(0), ptr(meta.q_start), ptr(meta.ctx_len), ptr(sinks),
+             meta.num_seqs, meta.max_q_len, H, G, d, vd, BS, float(scale), float(out_scale), k_cache.shape[0], dt)
     return out

@@ -146,3 +146,63 @@ def pool_l2norm(hidden: torch.Tensor, starts: torch.Tensor, lengths: torch.Tenso
 
 def softmax_scale(head_dim: int) -> float:
     return 1.0 / math.sqrt(head_dim)
+
+
+# ---------------------------------------------------------------------------------------------- partial rotary + value norm
+def rope_table(max_pos: int, rot_dims: int, base: float, device=None) -> torch.Tensor:
+    """[max_pos, rot_dims] fp32: cos(p f_i) in [:rot_dims/2], sin in [rot_dims/2:], f_i = base^(-2i/rot_dims);
+    angles formed in float64 and rounded once."""
+    i = torch.arange(rot_dims // 2, dtype=torch.float64)
+    f = torch.outer(torch.arange(max_pos, dtype=torch.float64), torch.as_tensor(base, dtype=torch.float64) ** (-2.0 * i / max(1, rot_dims)))
+    return torch.cat([f.cos(), f.sin()], dim=-1).float().to(device)
+
+
+def rope_vnorm_store(proj: torch.Tensor, qoff: int, koff: int, voff: int, positions: torch.Tensor,
+                     table: torch.Tensor, slot_mapping: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                     H: int, G: int, d: int, vd: int, rot_dims: int, eps: float) -> torch.Tensor:
+    """From a fused projection ``proj`` [T, ld] (q heads at column qoff, k at koff, v at voff): rotate the first
+    ``rot_dims`` dims of every q / k head (dim i paired with i + rot_dims/2), divide every v head by its root
+    mean square (fp32), store k / v into the paged caches k_cache [blocks, G, BS, d] / v_cache [blocks, G, BS, vd]
+    at ``slot_mapping`` (-1: not stored) and return q [T, H, d]."""
+    T = proj.shape[0]
+    BS = k_cache.shape[2]
+    if not proj.is_cuda:
+        x = proj.float()
+        q = x[:, qoff:qoff + H * d].reshape(T, H, d).clone()
+        k = x[:, koff:koff + G * d].reshape(T, G, d).clone()
+        v = x[:, voff:voff + G * vd].reshape(T, G, vd)
+        if rot_dims:
+            h2 = rot_dims // 2
+            cs = table[positions.long()]
+            c, s = cs[:, None, :h2], cs[:, None, h2:]
+            for t in (q, k):
+                a, b = t[..., :h2].clone(), t[..., h2:rot_dims].clone()
+                t[..., :h2] = a * c - b * s
+                t[..., h2:rot_dims] = b * c + a * s
+        v = v / torch.sqrt(v.pow(2).mean(-1, keepdim=True) + eps)
+        ok = slot_mapping >= 0
+        sl = slot_mapping[ok].long()
+        k_cache[sl // BS, :, sl % BS] = k[ok].to(k_cache.dtype)
+        v_cache[sl // BS, :, sl % BS] = v[ok].to(v_cache.dtype)
+        return q.to(proj.dtype)
+    assert proj.stride(1) == 1 and k_cache.dtype == proj.dtype and v_cache.dtype == proj.dtype
+    q = torch.empty(T, H, d, dtype=proj.dtype, device=proj.device)
+    call("grag_rope_vnorm_store", ptr(proj), proj.stride(0), qoff, koff, voff, ptr(positions), ptr(table),
+         table.shape[0], ptr(slot_mapping), ptr(q), ptr(k_cache), ptr(v_cache), T, H, G, d, vd, rot_dims, BS,
+         k_cache.shape[0] * BS, float(eps), 0 if proj.dtype == torch.bfloat16 else 1)
+    return q
+
+
+def clamped_glu(gu: torch.Tensor, limit: float, alpha: float = 1.702) -> torch.Tensor:
+    """gu [T, 2F] (gate | up) -> g sigmoid(alpha g) (u + 1) with g = min(gate, limit), u = clamp(up, +-limit)."""
+    T, F2 = gu.shape
+    F = F2 // 2
+    if not gu.is_cuda:
+        g = gu[:, :F].float().clamp(max=limit)
+        u = gu[:, F:].float().clamp(-limit, limit)
+        return (g * torch.sigmoid(alpha * g) * (u + 1.0)).to(gu.dtype)
+    assert gu.is_contiguous()
+    out = torch.empty(T, F, dtype=gu.dtype, device=gu.device)
+    call("grag_clamped_glu", ptr(gu), ptr(out), T, F, float(limit), float(alpha),
+         0 if gu.dtype == torch.bfloat16 else 1)
+    return out

@@ -137,3 +137,47 @@ def embed_gather(ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
     out = torch.empty(T, H, dtype=table.dtype, device=table.device)
     call("grag_embed_gather", ptr(ids), ptr(table), ptr(out), T, H, table.shape[0])
     return out
+
+
+# ---------------------------------------------------------------------------------------------- Dynamic Tanh
+def dyt_ref(x: torch.Tensor, alpha: float, w: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """Dynamic Tanh norm, fp32: tanh(alpha x) w + b (element-wise; no mean, no variance)."""
+    return torch.tanh(alpha * x.float()) * w.float() + b.float()
+
+
+def dyt_residual(resid: torch.Tensor, y: torch.Tensor | None = None, post=None, add_rows: torch.Tensor | None = None,
+                 add_vec: torch.Tensor | None = None, pre=None, out_dtype=torch.bfloat16) -> torch.Tensor | None:
+    """One pass over the fp32 residual stream ``resid`` [T, H] (updated in place):
+    resid += dyt_post(y) (+ add_rows [T, H] fp32) (+ add_vec [H] fp32), then returns dyt_pre(resid) in
+    ``out_dtype`` (None without ``pre``).  ``post`` / ``pre`` are (alpha, w fp32 [H], b fp32 [H]) triples:
+    the norm that closes one sublayer and the norm that opens the next, fused at the sublayer boundary."""
+    assert resid.dtype == torch.float32 and resid.is_contiguous()
+    T, H = resid.shape
+    if not _on_gpu(resid):
+        if y is not None:
+            resid += dyt_ref(y, *post)
+        if add_rows is not None:
+            resid += add_rows
+        if add_vec is not None:
+            resid += add_vec
+        return None if pre is None else dyt_ref(resid, *pre).to(out_dtype)
+    out = torch.empty(T, H, dtype=out_dtype, device=resid.device) if pre is not None else None
+    if y is not None:
+        assert y.dtype == out_dtype and y.is_contiguous() and y.shape == resid.shape
+    a1, w1, b1 = post if y is not None else (0.0, None, None)
+    a2, w2, b2 = pre if pre is not None else (0.0, None, None)
+    call("grag_dyt_residual", ptr(y), float(a1), ptr(w1), ptr(b1), ptr(resid), ptr(add_rows), ptr(add_vec), float(a2),
+         ptr(w2), ptr(b2), ptr(out), T, H, 0 if out_dtype == torch.bfloat16 else 1)
+    return out
+
+
+def embed_gather_f32(ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
+    """Embedding rows as an fp32 [T, H] residual stream (table bf16 or fp32)."""
+    if not _on_gpu(table):
+        return table[ids.long()].float()
+    ids = ids.to(torch.int32).contiguous()
+    T, H = ids.numel(), table.shape[1]
+    out = torch.empty(T, H, dtype=torch.float32, device=table.device)
+    call("grag_embed_f32", ptr(ids), ptr(table), ptr(out), T, H, table.shape[0],
+         0 if table.dtype == torch.bfloat16 else 1)
+    return out

@@ -1,0 +1,119 @@
+"""Recurrent sequence mixers with a carried fp32 state per sequence (HIP on device tensors, plain fp32 loops on
+CPU): linear attention with a fixed per-head decay, and the minGRU gated recurrence.
+
+State lives in slot-indexed pools ([slots, ...] fp32) owned by the engine; ``meta.state_slots`` [nseq] names each
+sequence's slot.  A sequence whose first token of the step is position 0 starts from a zero state (so a freed
+slot needs no reset when it is used again); otherwise the step continues from the slot's state and leaves the
+state after its last token there.  Tokens are consumed in order, so a prompt may be cut into steps anywhere.
+"""
+from __future__ import annotations
+
+import torch
+
+from ._lib import call, ptr
+from .attention import AttnMetadata
+
+
+def _dt(t: torch.Tensor) -> int:
+    return 0 if t.dtype == torch.bfloat16 else 1
+
+
+def _parts(meta: AttnMetadata):
+    """(meta, first row, end row) of a step's parts: prefill chunks, then the decode rows of a mixed step."""
+    dec = meta.extra.get("decode_rows")
+    if dec is None:
+        return [(meta, 0, meta.num_tokens)]
+    Tp, dmeta = dec
+    return [(meta, 0, Tp), (dmeta, Tp, Tp + dmeta.num_tokens)]
+
+
+def decay_attention(proj: torch.Tensor, qoff: int, koff: int, voff: int, decay: torch.Tensor, state: torch.Tensor,
+                    meta: AttnMetadata, H: int, d: int, vd: int) -> torch.Tensor:
+    """Linear attention with decay.  From the fused projection ``proj`` [T, ld]: q, k = silu(columns qoff / koff,
+    H x d), v = silu(columns voff, H x vd).  Per head S_t = decay_h S_(t-1) + k_t v_t^T (state [slots, H, d, vd]
+    fp32), o_t = S_t^T q_t.  Returns o [T, H*vd] fp32."""
+    T = proj.shape[0]
+    out = torch.empty(T, H * vd, dtype=torch.float32, device=proj.device)
+    for m, r0, r1 in _parts(meta):
+        if r1 <= r0:
+            continue
+        if not proj.is_cuda:
+            _decay_attention_cpu(proj[r0:r1], qoff, koff, voff, decay, state, m, H, d, vd, out[r0:r1])
+            continue
+        assert proj.stride(1) == 1 and state.dtype == torch.float32 and state.is_contiguous()
+        x = proj[r0:r1]
+        call("grag_decay_attn_scan", ptr(x), proj.stride(0), qoff, koff, voff, ptr(decay), ptr(state),
+             ptr(m.state_slots), ptr(m.q_start), ptr(m.ctx_len), ptr(out[r0:r1]), m.num_seqs, H, d, vd,
+             state.shape[0], _dt(proj))
+    return out
+
+
+def _decay_attention_cpu(x, qoff, koff, voff, decay, state, m, H, d, vd, out):
+    F = torch.nn.functional
+    qs, cl, sl = m.q_start.tolist(), m.ctx_len.tolist(), m.state_slots.tolist()
+    x = x.float()
+    for s in range(m.num_seqs):
+        a, b = qs[s], qs[s + 1]
+        if b <= a:
+            continue
+        S = torch.zeros(H, d, vd) if cl[s] - (b - a) == 0 else state[sl[s]].clone()
+        q = F.silu(x[a:b, qoff:qoff + H * d]).view(-1, H, d)
+        k = F.silu(x[a:b, koff:koff + H * d]).view(-1, H, d)
+        v = F.silu(x[a:b, voff:voff + H * vd]).view(-1, H, vd)
+        lam = decay.float().view(H, 1, 1)
+        for t in range(b - a):
+            S = lam * S + k[t, :, :, None] * v[t, :, None, :]
+            out[a + t] = torch.einsum("hdv,hd->hv", S, q[t]).reshape(-1)
+        state[sl[s]] = S
+
+
+def gated_rmsnorm(x: torch.Tensor, w: torch.Tensor, proj: torch.Tensor, goff: int, eps: float,
+                  out: torch.Tensor, out_scale: float = 1.0) -> torch.Tensor:
+    """out = out_scale * x / rms(x) * w * sigmoid(gate): x [T, N] fp32 normalised over the whole row, the gate
+    read from columns goff.. of the fused projection; ``out`` [T, N] may be a column slice of a wider buffer."""
+    T, N = x.shape
+    if not x.is_cuda:
+        g = torch.sigmoid(proj[:, goff:goff + N].float())
+        out.copy_((x / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + eps) * w.float() * g * out_scale))
+        return out
+    assert x.is_contiguous() and out.stride(1) == 1 and out.dtype == proj.dtype
+    call("grag_gated_rmsnorm", ptr(x), ptr(w), ptr(proj), proj.stride(0), goff, ptr(out), out.stride(0), T, N,
+         float(eps), float(out_scale), _dt(proj))
+    return out
+
+
+def mingru_scan(proj: torch.Tensor, zoff: int, xoff: int, goff: int, bz: torch.Tensor, bx: torch.Tensor,
+                state: torch.Tensor, meta: AttnMetadata, W: int) -> torch.Tensor:
+    """minGRU over a step's tokens.  From the fused projection [T, ld]: z = sigmoid(columns zoff + bz),
+    u = columns xoff + bx, candidate = u + 1/2 where u >= 0 else sigmoid(u);
+    S_t = (1 - z) S_(t-1) + z candidate (state [slots, W] fp32); returns S_t * silu(columns goff) [T, W]."""
+    T = proj.shape[0]
+    out = torch.empty(T, W, dtype=proj.dtype, device=proj.device)
+    for m, r0, r1 in _parts(meta):
+        if r1 <= r0:
+            continue
+        if not proj.is_cuda:
+            _mingru_cpu(proj[r0:r1].float(), zoff, xoff, goff, bz, bx, state, m, W, out[r0:r1])
+            continue
+        assert proj.stride(1) == 1 and state.dtype == torch.float32 and state.is_contiguous()
+        call("grag_mingru_scan", ptr(proj[r0:r1]), proj.stride(0), zoff, xoff, goff, ptr(bz), ptr(bx), ptr(state),
+             ptr(m.state_slots), ptr(m.q_start), ptr(m.ctx_len), ptr(out[r0:r1]), m.num_seqs, W, state.shape[0],
+             _dt(proj))
+    return out
+
+
+def _mingru_cpu(x, zoff, xoff, goff, bz, bx, state, m, W, out):
+    qs, cl, sl = m.q_start.tolist(), m.ctx_len.tolist(), m.state_slots.tolist()
+    z = torch.sigmoid(x[:, zoff:zoff + W] + bz.float())
+    u = x[:, xoff:xoff + W] + bx.float()
+    c = torch.where(u >= 0, u + 0.5, torch.sigmoid(u))
+    g = torch.nn.functional.silu(x[:, goff:goff + W])
+    for s in range(m.num_seqs):
+        a, b = qs[s], qs[s + 1]
+        if b <= a:
+            continue
+        S = torch.zeros(W) if cl[s] - (b - a) == 0 else state[sl[s]].clone()
+        for t in range(a, b):
+            S = (1.0 - z[t]) * S + z[t] * c[t]
+            out[t] = (S * g[t]).to(out.dtype)
+        state[sl[s]] = S

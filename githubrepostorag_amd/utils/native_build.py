@@ -40,6 +40,10 @@ HIPCC_FLAGS = [
     "-ffp-contract=fast",
     "-munsafe-fp-atomics",
     "-Wno-unused-result",
+    # no packed-fp32 VALU forms (v_pk_fma_f32 and friends): some of them have returned wrong values on this
+    # hardware; -O3 would otherwise form them from plain float code.  (The host pass warns that it does not
+    # know the feature: harmless.)
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
 CXX_FLAGS = ["-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function"]
 
