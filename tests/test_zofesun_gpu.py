@@ -1,0 +1,123 @@
+"""Zofesun on the HIP kernels (cuda:0): every mechanism alone and the engine scenarios of zofesun_cases.py
+against the float64 oracle -- in fp32 (the kernels' 32-bit parts are then the whole computation: tight bounds)
+and in bf16 (the serving precision)."""
+import pytest
+import torch
+
+import test_zofesun as T
+import zofesun_cases as C
+
+pytestmark = pytest.mark.gpu
+
+F32 = 5e-5   # fp32 GEMMs + fp32 kernels against float64
+BF16 = 0.06  # bf16 GEMMs and activations
+
+
+@pytest.fixture(autouse=True)
+def _true_fp32():
+    torch.backends.cuda.matmul.allow_tf32 = False
+    yield
+
+
+def test_kernel_library_is_loaded():
+    from githubrepostorag_amd.ops import _lib
+
+    assert _lib.lib() is not None and _lib.loaded_path()
+    assert hasattr(_lib.lib(), "grag_sink_attn_prefill") and hasattr(_lib.lib(), "grag_mingru_scan")
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-5), (torch.bfloat16, 0.03)])
+def test_sink_attention_far_keys_and_page_borders(dtype, tol):
+    T.sink_attention_case("cuda", dtype, tol)
+    T.sink_attention_case("cuda", dtype, tol, T=67, far=(0, 3, 4, 63, 64), bs=4)
+
+
+def test_sink_attention_wide_heads():
+    """Head sizes past one 64-lane pass, and a key tile that does not fit 64 keys."""
+    from githubrepostorag_amd.ops.attention import AttnMetadata, sink_attention
+    import zofesun_oracle as O
+
+    g = torch.Generator().manual_seed(4)
+    for (H, G, d, vd, n) in ((2, 1, 200, 136, 70), (3, 3, 256, 256, 40)):
+        q, k, v = (torch.randn(n, H, d, generator=g) * 0.2, torch.randn(n, G, d, generator=g) * 0.2,
+                   torch.randn(n, G, vd, generator=g))
+        sinks = torch.randn(H, generator=g)
+        want = O.sink_attention(q.double(), k.double(), v.double(), 0.5, sinks.double())
+        kc, vc, bt, _ = T._paged(k, v, 16)
+        i32 = dict(dtype=torch.int32, device="cuda")
+        for a in (0, n - 1):
+            m = n - a
+            meta = AttnMetadata(q_start=torch.tensor([0, m], **i32), ctx_len=torch.tensor([n], **i32),
+                                block_tables=bt.cuda(), slot_mapping=None, max_q_len=m, num_seqs=1, num_tokens=m,
+                                is_decode=(m == 1))
+            got = sink_attention(q[a:].cuda().contiguous(), kc.cuda(), vc.cuda(), meta, 0.5, sinks.cuda())
+            assert float((got.double().cpu().view(m, H, vd) - want[a:]).abs().max()) < 2e-5
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-5), (torch.bfloat16, 2e-5)])
+def test_recurrent_mixers_alone(dtype, tol):
+    T.recurrent_case("cuda", dtype, tol)  # (bf16 inputs are rounded before both sides: the recurrences are fp32)
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-5), (torch.bfloat16, 0.03)])
+def test_elementwise_mechanisms_alone(dtype, tol):
+    T.elementwise_case("cuda", dtype, tol)
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, F32), (torch.bfloat16, BF16)])
+def test_whole_prompt_and_layer_taps(dtype, tol):
+    C.case_whole_and_layers("cuda", tol, dtype)
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, F32), (torch.bfloat16, BF16)])
+def test_prefill_against_decode(dtype, tol):
+    C.case_prefill_vs_decode("cuda", tol, dtype)
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, F32), (torch.bfloat16, BF16)])
+def test_portions(dtype, tol):
+    C.case_portions("cuda", tol, dtype)
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, F32), (torch.bfloat16, BF16)])
+def test_unequal_batches(dtype, tol):
+    C.case_batches("cuda", tol, dtype)
+
+
+def test_pages_and_slots_used_again():
+    C.case_reuse("cuda", F32)
+
+
+def test_other_sizes():
+    C.case_other_sizes("cuda", F32)
+    C.case_other_sizes("cuda", BF16, torch.bfloat16)
+
+
+def test_first_tokens():
+    C.case_first_tokens("cuda", F32)
+
+
+def test_long_decode():
+    C.case_long_decode("cuda", F32)
+
+
+@pytest.mark.parametrize("graphs,mixed,window,max_batched", [(False, False, 1, 4096), (True, False, 1, 4096),
+                                                             (True, False, 4, 4096), (False, True, 1, 8)])
+def test_greedy_generation(graphs, mixed, window, max_batched):
+    C.case_generate("cuda", graphs=graphs, mixed=mixed, window=window, max_batched=max_batched)
+
+
+def test_bf16_batch_invariance():
+    """bf16 serving: a request's logits beside other requests equal its logits alone (the same kernels see the
+    same operands per row; only GEMM tiling may differ with the batch's row count)."""
+    import numpy as np
+    import zofesun_oracle as O
+
+    cfg = O.make_config()
+    sd = O.make_weights(cfg, seed=37)
+    a, b = C.tokens(cfg, 40, 1), C.tokens(cfg, 13, 2)
+    _, eng = C.build(cfg, sd, "cuda", torch.bfloat16)
+    alone = C.feed_in_portions(eng, "a", a, [40])
+    o1 = eng.feed([("a2", a[:25], list(range(25))), ("b", b[:12], [])], [])
+    o2 = eng.feed([("a2", a[25:], list(range(15))), ("b", b[12:], [0])], ["a2", "b"])
+    assert C.rel_err(np.concatenate([o1, o2[:15]], 0), alone) < 0.02
