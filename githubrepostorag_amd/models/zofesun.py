@@ -134,7 +134,11 @@ class ZofesunModel:
         expect("embed", cfg.vocab_size, H)
         expect("head", cfg.vocab_size, H)
         self.embed = act("embed")
-        self.head = act("head")
+        # LM head rows padded to a multiple of 8: the sampler reads logit rows 8 at a time (zero rows, cut off
+        # again in compute_logits)
+        pad = -cfg.vocab_size % 8
+        self.head = act("head") if not pad else torch.cat(
+            [act("head"), torch.zeros(pad, H, dtype=dt, device=dev)], 0).contiguous()
         self.final_norm = norm("final.norm")
         self.loop_step = None
         if cfg.loop_stop > cfg.loop_start:
@@ -297,5 +301,5 @@ class ZofesunModel:
         return dyt_residual(x, y, post, pre=self.final_norm, out_dtype=dt)
 
     def compute_logits(self, hidden: torch.Tensor) -> torch.Tensor:
-        """final-normed hidden [B, H] -> logits [B, vocab]."""
-        return linear(hidden, self.head)
+        """final-normed hidden [B, H] -> logits [B, vocab] (a view of the padded GEMM output)."""
+        return linear(hidden, self.head)[:, : self.cfg.vocab_size]
