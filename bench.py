@@ -174,6 +174,9 @@ def parse():
     ap.add_argument("--recall-queries", type=int, default=64,
                     help="queries per rank for recall@top-k of the IVF search vs an exact scan of every shard "
                          "(index_recall; 0: skip)")
+    ap.add_argument("--hybrid", action="store_true",
+                    help="instead of the headline workload: prefill / decode throughput of the Zofesun hybrid decoder "
+                         "beside the equal-size Qwen2 decoder, and a per-kernel roofline table (one GPU)")
     ap.add_argument("--out", default=None)
     args = ap.parse_args()
     if args.preset:
@@ -239,6 +242,15 @@ def spawn_ranks(n: int) -> int:
 
 def main():
     args = parse()
+    if args.hybrid:  # the hybrid decoder beside the equal-size Qwen2 decoder (engine/bench_hybrid.py); one GPU
+        from githubrepostorag_amd.engine.bench_hybrid import run as run_hybrid
+
+        res = run_hybrid(args)
+        if args.out:
+            with open(args.out, "w") as f:
+                json.dump(res, f, indent=1)
+        print(json.dumps(res))
+        return
     if args.gpus > 1 and "WORLD_SIZE" not in os.environ:
         sys.exit(spawn_ranks(args.gpus))
     if args.switch_interval > 0:

@@ -237,6 +237,257 @@ sink_attn_prefill_kernel(const T* __restrict__ q, const T* __restrict__ k_cache,
   }
 }
 
+// prefill on the matrix cores (bf16 activations, d and vd multiples of 16): grid (tiles of 64 queries, H, nseq), 4 waves
+// of 16 queries.  Per 64-key tile (K [64][d+8] and V^T [vd][64+4] staged in LDS as bf16):
+//   S^T = K Q^T      v_mfma_f32_16x16x16_bf16: bf16 products are exact in fp32, fp32 accumulation; the C fragment
+//                    (rows = keys 4*(lane/16)+i, column = query lane%16) is the B fragment of the next product,
+//   softmax in fp32  per query = per lane column: max / sum over the fragment's rows and the 4 lane quads,
+//   O^T += V^T P^T   with the fp32 weights split into bf16 hi + lo parts (two products): 16 mantissa bits of P
+//                    reach the accumulator, below the bf16 rounding of V and of the stored output.
+template <int NKM, int NVM>
+__global__ void __launch_bounds__(256)
+sink_attn_prefill_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_cache,
+                              const bf16* __restrict__ v_cache, bf16* __restrict__ out, int out_ld,
+                              const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ q_start,
+                              const int* __restrict__ ctx_len, const float* __restrict__ sinks, int H, int G, int d,
+                              int vd, int BS, float scale, float out_scale, int nblocks) {
+  constexpr int KT = 64;
+  extern __shared__ __attribute__((aligned(16))) char smem_raw[];
+  const int seq = blockIdx.z, h = blockIdx.y, g = h / (H / G);
+  const int qa = q_start[seq], qlen = q_start[seq + 1] - qa, ctx = ctx_len[seq];
+  const int q0 = blockIdx.x * 64;
+  if (q0 >= qlen) return;
+  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+  const int ql = lane & 15, quad = lane >> 4;
+  const int nk = d >> 4, nv = vd >> 4;
+  const int kstride = d + 8, vstride = KT + 4;
+  short* Ks = reinterpret_cast<short*>(smem_raw);  // [KT][d+8] bf16 bits
+  short* Vt = Ks + KT * kstride;                   // [vd][KT+4]
+  const int tq = q0 + wid * 16 + ql;               // this lane's query (a fragment column)
+  const bool q_ok = tq < qlen;
+  bf16x4_t qf[NKM];
+#pragma unroll
+  for (int ks = 0; ks < NKM; ++ks) {
+    qf[ks] = bf16x4_t{0, 0, 0, 0};
+    if (ks < nk && q_ok)
+      qf[ks] = *reinterpret_cast<const bf16x4_t*>(q + ((size_t)(qa + tq) * H + h) * d + ks * 16 + quad * 4);
+  }
+  const int pos0 = ctx - qlen;
+  const int qpos = pos0 + tq;
+  float m = sinks[h], l = 1.f;
+  f32x4_t acc[NVM];
+#pragma unroll
+  for (int v = 0; v < NVM; ++v) acc[v] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  const int nkeys = min(ctx, pos0 + min(q0 + 64, qlen));
+  const int wave_qmax = pos0 + min(q0 + wid * 16 + 15, qlen - 1);
+  const int* bt = block_tables + (size_t)seq * bt_stride;
+  const int dv8 = d >> 3, vv8 = vd >> 3;
+  for (int k0 = 0; k0 < nkeys; k0 += KT) {
+    __syncthreads();
+    const int kn = min(KT, nkeys - k0);
+    for (int idx = threadIdx.x; idx < KT * dv8; idx += 256) {
+      const int kk = idx / dv8, c = idx - kk * dv8;
+      bf16x8_t v = bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
+      if (kk < kn) {
+        const int key = k0 + kk;
+        const int blk = bt[key / BS];
+        if (index_ok(blk, nblocks, ERR_BLOCK_PREFILL))
+          v = *reinterpret_cast<const bf16x8_t*>(k_cache + (((size_t)blk * G + g) * BS + key % BS) * d + c * 8);
+      }
+      *reinterpret_cast<bf16x8_t*>(Ks + kk * kstride + c * 8) = v;
+    }
+    for (int idx = threadIdx.x; idx < KT * vv8; idx += 256) {
+      const int kk = idx / vv8, c = idx - kk * vv8;
+      bf16x8_t v = bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
+      if (kk < kn) {
+        const int key = k0 + kk;
+        const int blk = bt[key / BS];
+        if (blk >= 0 && blk < nblocks)
+          v = *reinterpret_cast<const bf16x8_t*>(v_cache + (((size_t)blk * G + g) * BS + key % BS) * vd + c * 8);
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) Vt[(c * 8 + e) * vstride + kk] = v[e];
+    }
+    __syncthreads();
+    if (k0 > wave_qmax) continue;  // every key of the tile lies after this wave's queries
+    f32x4_t st[4];
+#pragma unroll
+    for (int n = 0; n < 4; ++n) {
+      st[n] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < NKM; ++ks) {
+        if (ks < nk) {
+          const bf16x4_t a = *reinterpret_cast<const bf16x4_t*>(Ks + (16 * n + ql) * kstride + ks * 16 + quad * 4);
+          st[n] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, qf[ks], st[n], 0, 0, 0);
+        }
+      }
+    }
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int n = 0; n < 4; ++n)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = k0 + 16 * n + 4 * quad + i;
+        const bool vis = q_ok && key < nkeys && key <= qpos;
+        const float sc = vis ? st[n][i] * scale : -INFINITY;
+        st[n][i] = sc;
+        tmax = fmaxf(tmax, sc);
+      }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    const float mn = fmaxf(m, tmax);  // finite: m starts at the sink
+    const float alpha = expf(m - mn);
+    float psum = 0.f;
+#pragma unroll
+    for (int n = 0; n < 4; ++n)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float p = st[n][i] == -INFINITY ? 0.f : expf(st[n][i] - mn);
+        st[n][i] = p;
+        psum += p;
+      }
+    psum += __shfl_xor(psum, 16, 64);
+    psum += __shfl_xor(psum, 32, 64);
+    l = l * alpha + psum;
+    m = mn;
+#pragma unroll
+    for (int v = 0; v < NVM; ++v) acc[v] *= alpha;
+#pragma unroll
+    for (int n = 0; n < 4; ++n) {
+      bf16x4_t ph, pl;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const short hi = f2bits(st[n][j]);
+        ph[j] = hi;
+        pl[j] = f2bits(st[n][j] - bits2f(hi));
+      }
+#pragma unroll
+      for (int v = 0; v < NVM; ++v) {
+        if (v < nv) {
+          const bf16x4_t a = *reinterpret_cast<const bf16x4_t*>(Vt + (16 * v + ql) * vstride + 16 * n + 4 * quad);
+          acc[v] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, ph, acc[v], 0, 0, 0);
+          acc[v] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, pl, acc[v], 0, 0, 0);
+        }
+      }
+    }
+  }
+  if (q_ok) {
+    const float r = out_scale / l;
+    bf16* orow = out + (size_t)(qa + tq) * out_ld + h * vd;
+#pragma unroll
+    for (int v = 0; v < NVM; ++v) {
+      if (v < nv) {
+        bf16x4_t o;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[i] = f2bits(acc[v][i] * r);
+        *reinterpret_cast<bf16x4_t*>(orow + 16 * v + 4 * quad) = o;
+      }
+    }
+  }
+}
+
+// decode, bf16 with d % 8 == 0 and vd even: as the kernel below, with 16-byte K loads (lane = key) and 4-byte V
+// loads (lane = a pair of value dims).
+__global__ void __launch_bounds__(256)
+sink_attn_decode_vec_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_cache,
+                            const bf16* __restrict__ v_cache, bf16* __restrict__ out, int out_ld,
+                            const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ ctx_len,
+                            const float* __restrict__ sinks, int H, int G, int d, int vd, int BS, float scale,
+                            float out_scale, int nblocks) {
+  extern __shared__ float smem[];
+  const int seq = blockIdx.y, h = blockIdx.x, g = h / (H / G);
+  const int ctx = ctx_len[seq];
+  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+  float* Qs = smem;               // [d]
+  float* Ps = Qs + d;             // [4][64]
+  float* Ms = Ps + 4 * 64;        // [4] m, [4] l
+  float* As = Ms + 8;             // [4][vd]
+  for (int i = threadIdx.x; i < d; i += 256) Qs[i] = (float)q[((size_t)seq * H + h) * d + i];
+  __syncthreads();
+  float m = wid == 0 ? sinks[h] : -INFINITY, l = wid == 0 ? 1.f : 0.f;
+  constexpr int VC = 2;  // pairs of value dims per lane: vd <= 256
+  float acc[VC][2];
+#pragma unroll
+  for (int c = 0; c < VC; ++c) acc[c][0] = acc[c][1] = 0.f;
+  const int* bt = block_tables + (size_t)seq * bt_stride;
+  float* pw = Ps + wid * 64;
+  const int ntiles = (ctx + 63) >> 6;
+  const int d8 = d >> 3;
+  for (int t = wid; t < ntiles; t += 4) {
+    const int key = t * 64 + lane;
+    const bool vis = key < ctx;
+    float s = 0.f;
+    if (vis) {
+      int blk = bt[key / BS];
+      if (!index_ok(blk, nblocks, ERR_BLOCK_DECODE)) blk = 0;
+      const bf16x8_t* kr = reinterpret_cast<const bf16x8_t*>(k_cache + (((size_t)blk * G + g) * BS + key % BS) * d);
+      for (int c = 0; c < d8; ++c) {
+        const bf16x8_t kv = kr[c];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) s = fmaf(Qs[c * 8 + e], bits2f(kv[e]), s);
+      }
+    }
+    const float sc = vis ? s * scale : -INFINITY;
+    const float mn = fmaxf(m, wave_max(sc));
+    const float p = vis ? expf(sc - mn) : 0.f;
+    const float alpha = (m == -INFINITY) ? 0.f : expf(m - mn);
+    l = l * alpha + wave_sum(p);
+    m = mn;
+    pw[lane] = p;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    const int kn = min(64, ctx - t * 64);
+#pragma unroll
+    for (int c = 0; c < VC; ++c) {
+      const int j = 2 * lane + 128 * c;
+      float a0 = acc[c][0] * alpha, a1 = acc[c][1] * alpha;
+      if (j < vd) {
+        for (int kk = 0; kk < kn; ++kk) {
+          const int key2 = t * 64 + kk;
+          int b2 = bt[key2 / BS];
+          if (b2 < 0 || b2 >= nblocks) b2 = 0;
+          const uint32_t w = *reinterpret_cast<const uint32_t*>(v_cache + (((size_t)b2 * G + g) * BS + key2 % BS) * vd + j);
+          const float pk = pw[kk];
+          a0 = fmaf(pk, __uint_as_float(w << 16), a0);
+          a1 = fmaf(pk, __uint_as_float(w & 0xffff0000u), a1);
+        }
+      }
+      acc[c][0] = a0;
+      acc[c][1] = a1;
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+  if (lane == 0) {
+    Ms[wid] = m;
+    Ms[4 + wid] = l;
+  }
+#pragma unroll
+  for (int c = 0; c < VC; ++c) {
+    const int j = 2 * lane + 128 * c;
+    if (j < vd) {
+      As[wid * vd + j] = acc[c][0];
+      As[wid * vd + j + 1] = acc[c][1];
+    }
+  }
+  __syncthreads();
+  if (wid == 0) {
+    float M = Ms[0];
+    for (int w = 1; w < 4; ++w) M = fmaxf(M, Ms[w]);
+    float L = 0.f, f[4];
+    for (int w = 0; w < 4; ++w) {
+      f[w] = Ms[w] == -INFINITY ? 0.f : expf(Ms[w] - M);
+      L += Ms[4 + w] * f[w];
+    }
+    const float r = out_scale / L;
+    for (int j = lane; j < vd; j += 64) {
+      float o = 0.f;
+      for (int w = 0; w < 4; ++w) o += As[w * vd + j] * f[w];
+      out[(size_t)seq * out_ld + h * vd + j] = (bf16)(o * r);
+    }
+  }
+}
+
 // decode (one query token per sequence): grid (H, nseq), 256 threads.  Each of the 4 waves walks every 4th
 // 64-key tile (lane = key, K rows read from the cache), keeps its own (m, l, acc); the waves merge through LDS.
 template <typename T>
@@ -335,26 +586,47 @@ sink_attn_decode_kernel(const T* __restrict__ q, const T* __restrict__ k_cache, 
 // Per head: S_t = decay_h S_(t-1) + k_t v_t^T, o_t = S_t^T q_t, with q, k, v = silu(projection) and S [d, vd] fp32.
 // grid (H, nseq); thread j < vd owns column j of S in registers (DMAX rows).  Tokens of the launch are walked in
 // order, TB at a time through LDS.  Serves prefill chunks (qlen tokens) and decode rows (qlen = 1) alike.
-template <typename T, int DMAX>
+//
+// Long portions are cut into chunks of DECAY_CHUNK tokens that run side by side (MODE 1 -> prefix kernel -> MODE 2):
+//   MODE 0  the whole portion in one workgroup, from and to the slot's state (short portions, decode rows);
+//   MODE 1  grid.z = chunk: the chunk's own contribution U_c = sum_s decay^(len-1-s) k_s v_s^T from a zero state,
+//           written to the workspace ws [nseq * maxchunks, H, d, vd];
+//   (decay_chunk_prefix_kernel turns ws[c] into the state at the START of chunk c and stores the final state;)
+//   MODE 2  grid.z = chunk: outputs of the chunk's tokens, from the chunk-start state in ws.
+// Mathematically the same recurrence; only fp32 rounding differs with the cut.
+constexpr int DECAY_CHUNK = 64;
+
+template <typename T, int DMAX, int MODE>
 __global__ void decay_attn_scan_kernel(const T* __restrict__ proj, int ld, int qoff, int koff, int voff,
                                        const float* __restrict__ decay, float* __restrict__ state,
                                        const int* __restrict__ slots, const int* __restrict__ q_start,
                                        const int* __restrict__ ctx_len, float* __restrict__ out, int H, int d, int vd,
-                                       int nslots) {
+                                       int nslots, float* __restrict__ ws, int maxchunks) {
   constexpr int TB = 16;
   extern __shared__ float smem[];  // [TB][2][d]
   const int seq = blockIdx.y, h = blockIdx.x;
-  const int qa = q_start[seq], qlen = q_start[seq + 1] - qa;
+  int qa = q_start[seq], qlen = q_start[seq + 1] - qa;
   if (qlen <= 0) return;
   const int j = threadIdx.x;
   const bool fresh = ctx_len[seq] - qlen == 0;
-  const int slot = slots[seq];
-  const bool slot_ok = index_ok(slot, nslots, ERR_SAMPLER_SLOT);
+  const int slot = MODE == 0 ? slots[seq] : 0;
+  const bool slot_ok = MODE == 0 ? index_ok(slot, nslots, ERR_SAMPLER_SLOT) : true;
   float* Sg = state + (((size_t)(slot_ok ? slot : 0) * H + h) * d) * vd;
+  if (MODE != 0) {
+    const int c = blockIdx.z;
+    if (c * DECAY_CHUNK >= qlen) return;
+    qa += c * DECAY_CHUNK;
+    qlen = min(DECAY_CHUNK, qlen - c * DECAY_CHUNK);
+    Sg = ws + (((size_t)(seq * maxchunks + c) * H + h) * d) * vd;
+  }
   const float lam = decay[h];
   float S[DMAX];
 #pragma unroll
-  for (int i = 0; i < DMAX; ++i) S[i] = (!fresh && slot_ok && i < d && j < vd) ? Sg[(size_t)i * vd + j] : 0.f;
+  for (int i = 0; i < DMAX; ++i) {
+    if (MODE == 0) S[i] = (!fresh && slot_ok && i < d && j < vd) ? Sg[(size_t)i * vd + j] : 0.f;
+    if (MODE == 1) S[i] = 0.f;
+    if (MODE == 2) S[i] = (i < d && j < vd) ? Sg[(size_t)i * vd + j] : 0.f;
+  }
   for (int t0 = 0; t0 < qlen; t0 += TB) {
     const int nb = min(TB, qlen - t0);
     __syncthreads();
@@ -376,17 +648,46 @@ __global__ void decay_attn_scan_kernel(const T* __restrict__ proj, int ld, int q
         for (int i = 0; i < DMAX; ++i) {
           if (i < d) {
             S[i] = fmaf(lam, S[i], ks[i] * vj);
-            o = fmaf(S[i], qs[i], o);
+            if (MODE != 1) o = fmaf(S[i], qs[i], o);
           }
         }
-        out[tok * (size_t)(H * vd) + h * vd + j] = o;
+        if (MODE != 1) out[tok * (size_t)(H * vd) + h * vd + j] = o;
       }
     }
   }
-  if (slot_ok && j < vd) {
+  if (MODE != 2 && slot_ok && j < vd) {
 #pragma unroll
     for (int i = 0; i < DMAX; ++i)
       if (i < d) Sg[(size_t)i * vd + j] = S[i];
+  }
+}
+
+// ws[seq, c] (chunk c's own contribution) -> the state at the start of chunk c; the slot's state <- the state after
+// the last chunk.  grid (H, nseq), threads stride over the d * vd elements.
+__global__ void decay_chunk_prefix_kernel(const float* __restrict__ decay, float* __restrict__ state,
+                                          const int* __restrict__ slots, const int* __restrict__ q_start,
+                                          const int* __restrict__ ctx_len, float* __restrict__ ws, int maxchunks,
+                                          int H, int d, int vd, int nslots) {
+  const int seq = blockIdx.y, h = blockIdx.x;
+  const int qlen = q_start[seq + 1] - q_start[seq];
+  if (qlen <= 0) return;
+  const bool fresh = ctx_len[seq] - qlen == 0;
+  const int slot = slots[seq];
+  if (!index_ok(slot, nslots, ERR_SAMPLER_SLOT)) return;
+  float* Sg = state + ((size_t)slot * H + h) * d * vd;
+  const float lam = decay[h];
+  const int nch = (qlen + DECAY_CHUNK - 1) / DECAY_CHUNK;
+  const float full = powf(lam, (float)DECAY_CHUNK), last = powf(lam, (float)(qlen - (nch - 1) * DECAY_CHUNK));
+  const size_t cs = (size_t)H * d * vd;
+  for (int e = threadIdx.x; e < d * vd; e += blockDim.x) {
+    float S = fresh ? 0.f : Sg[e];
+    float* w = ws + ((size_t)seq * maxchunks * H + h) * d * vd + e;
+    for (int c = 0; c < nch; ++c) {
+      const float u = w[c * cs];
+      w[c * cs] = S;
+      S = fmaf(c == nch - 1 ? last : full, S, u);
+    }
+    Sg[e] = S;
   }
 }
 
@@ -435,6 +736,52 @@ __global__ void mingru_scan_kernel(const T* __restrict__ proj, int ld, int zoff,
     stf(out + (size_t)(qa + t) * W + c, S * silu_acc(ldf(row + goff + c)));
   }
   if (slot_ok) *sp = S;
+}
+
+// Long portions, chunks of MINGRU_CHUNK tokens side by side.  The recurrence is affine in the state, so a chunk
+// composes to S_end = A S_start + B with A = prod (1 - z_t) and B = its result from a zero state.
+//   pass 1 (PASS = 1): every (sequence, chunk, channel) writes its (A, B) to ws [nseq * maxchunks, 2, W];
+//   pass 2 (PASS = 2): every chunk folds the (A, B) of the chunks before it onto the slot's state (<= maxchunks
+//                      steps), then walks its tokens again and writes the outputs; the last chunk stores the state.
+constexpr int MINGRU_CHUNK = 64;
+
+template <typename T, int PASS>
+__global__ void mingru_chunk_kernel(const T* __restrict__ proj, int ld, int zoff, int xoff, int goff,
+                                    const float* __restrict__ bz, const float* __restrict__ bx,
+                                    float* __restrict__ state, const int* __restrict__ slots,
+                                    const int* __restrict__ q_start, const int* __restrict__ ctx_len,
+                                    T* __restrict__ out, int W, int nslots, float* __restrict__ ws, int maxchunks) {
+  const int seq = blockIdx.y, ch = blockIdx.z;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  const int qa = q_start[seq], qlen = q_start[seq + 1] - qa;
+  const int t0 = ch * MINGRU_CHUNK;
+  if (c >= W || t0 >= qlen) return;
+  const int n = min(MINGRU_CHUNK, qlen - t0);
+  const float zb = bz[c], xb = bx[c];
+  float* w = ws + (size_t)seq * maxchunks * 2 * W;
+  float S = 0.f, A = 1.f;
+  if (PASS == 2) {
+    const int slot = slots[seq];
+    const bool slot_ok = index_ok(slot, nslots, ERR_SAMPLER_SLOT);
+    S = (ctx_len[seq] - qlen == 0 || !slot_ok) ? 0.f : state[(size_t)slot * W + c];
+    for (int k = 0; k < ch; ++k) S = fmaf(w[(size_t)k * 2 * W + c], S, w[(size_t)k * 2 * W + W + c]);
+  }
+  for (int t = 0; t < n; ++t) {
+    const T* row = proj + (size_t)(qa + t0 + t) * ld;
+    const float z = sigmoid_acc(ldf(row + zoff + c) + zb);
+    const float u = ldf(row + xoff + c) + xb;
+    const float cand = u >= 0.f ? u + 0.5f : sigmoid_acc(u);
+    S = (1.f - z) * S + z * cand;
+    if (PASS == 1) A *= 1.f - z;
+    if (PASS == 2) stf(out + (size_t)(qa + t0 + t) * W + c, S * silu_acc(ldf(row + goff + c)));
+  }
+  if (PASS == 1) {
+    w[(size_t)ch * 2 * W + c] = A;
+    w[(size_t)ch * 2 * W + W + c] = S;
+  } else if (t0 + n == qlen) {
+    const int slot = slots[seq];
+    if (slot >= 0 && slot < nslots) state[(size_t)slot * W + c] = S;
+  }
 }
 
 // ------------------------------------------------------------------------------------------------ clamped GLU
@@ -509,6 +856,30 @@ GRAG_API hipError_t grag_sink_attn_prefill(const void* q, const void* k_cache, c
                                            int dt, hipStream_t st) {
   if (nseq <= 0 || max_q_len <= 0) return hipSuccess;
   if (vd > 64 * SA_VC || G <= 0 || H % G) return hipErrorInvalidValue;
+  if (dt == 0 && max_q_len >= 16 && d % 16 == 0 && vd % 16 == 0 && d <= 256 && vd <= 256 && out_ld % 4 == 0 &&
+      (reinterpret_cast<uintptr_t>(out) & 7) == 0 && (reinterpret_cast<uintptr_t>(q) & 7) == 0) {
+    const size_t mb = ((size_t)64 * (d + 8) + (size_t)vd * (64 + 4)) * sizeof(short);
+    const dim3 mgrid((max_q_len + 63) / 64, H, nseq);
+#define SA_MFMA(NK, NV)                                                                                              \
+  {                                                                                                                  \
+    if (mb > 48 * 1024) {                                                                                            \
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&sink_attn_prefill_mfma_kernel<NK, NV>),      \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)mb);                       \
+      if (e != hipSuccess) return e;                                                                                 \
+    }                                                                                                                \
+    hipLaunchKernelGGL((sink_attn_prefill_mfma_kernel<NK, NV>), mgrid, dim3(256), mb, st, (const bf16*)q,            \
+                       (const bf16*)k_cache, (const bf16*)v_cache, (bf16*)out, out_ld, block_tables, bt_stride,      \
+                       q_start, ctx_len, sinks, H, G, d, vd, BS, scale, out_scale, nblocks);                         \
+  }
+    const int nk = d / 16, nv = vd / 16;
+    if (nk <= 4 && nv <= 4) SA_MFMA(4, 4)
+    else if (nk <= 8 && nv <= 8) SA_MFMA(8, 8)
+    else if (nk <= 8) SA_MFMA(8, 16)
+    else if (nv <= 8) SA_MFMA(16, 8)
+    else SA_MFMA(16, 16)
+#undef SA_MFMA
+    return hipGetLastError();
+  }
   size_t bytes;
   const int KT = sa_key_tile(d, vd, &bytes);
   if (bytes > 160 * 1024) return hipErrorInvalidValue;
@@ -533,22 +904,29 @@ GRAG_API hipError_t grag_sink_attn_decode(const void* q, const void* k_cache, co
   if (nseq <= 0) return hipSuccess;
   if (vd > 64 * SA_VC || G <= 0 || H % G) return hipErrorInvalidValue;
   const size_t bytes = ((size_t)d + 4 * 64 + 8 + 4 * (size_t)vd) * sizeof(float);
+  if (dt == 0 && d % 8 == 0 && vd % 2 == 0 && vd <= 256) {
+    hipLaunchKernelGGL(sink_attn_decode_vec_kernel, dim3(H, nseq), dim3(256), bytes, st, (const bf16*)q,
+                       (const bf16*)k_cache, (const bf16*)v_cache, (bf16*)out, out_ld, block_tables, bt_stride,
+                       ctx_len, sinks, H, G, d, vd, BS, scale, out_scale, nblocks);
+    return hipGetLastError();
+  }
   DT_DISPATCH(dt, hipLaunchKernelGGL(sink_attn_decode_kernel<T>, dim3(H, nseq), dim3(256), bytes, st, (const T*)q,
                                      (const T*)k_cache, (const T*)v_cache, (T*)out, out_ld, block_tables, bt_stride,
                                      ctx_len, sinks, H, G, d, vd, BS, scale, out_scale, nblocks);)
   return hipGetLastError();
 }
 
-template <typename T>
+template <typename T, int MODE>
 static hipError_t launch_decay_scan(const T* proj, int ld, int qoff, int koff, int voff, const float* decay,
                                     float* state, const int* slots, const int* q_start, const int* ctx_len, float* out,
-                                    int nseq, int H, int d, int vd, int nslots, hipStream_t st) {
+                                    int nseq, int H, int d, int vd, int nslots, float* ws, int maxchunks,
+                                    hipStream_t st) {
   const int threads = ((vd + 63) / 64) * 64;
   const size_t bytes = (size_t)16 * 2 * d * sizeof(float);
-  const dim3 grid(H, nseq);
-#define DECAY_LAUNCH(DM)                                                                                          \
-  hipLaunchKernelGGL((decay_attn_scan_kernel<T, DM>), grid, dim3(threads), bytes, st, proj, ld, qoff, koff, voff, \
-                     decay, state, slots, q_start, ctx_len, out, H, d, vd, nslots)
+  const dim3 grid(H, nseq, MODE == 0 ? 1 : maxchunks);
+#define DECAY_LAUNCH(DM)                                                                                     \
+  hipLaunchKernelGGL((decay_attn_scan_kernel<T, DM, MODE>), grid, dim3(threads), bytes, st, proj, ld, qoff, koff, \
+                     voff, decay, state, slots, q_start, ctx_len, out, H, d, vd, nslots, ws, maxchunks)
   if (d <= 16) {
     DECAY_LAUNCH(16);
   } else if (d <= 32) {
@@ -564,14 +942,30 @@ static hipError_t launch_decay_scan(const T* proj, int ld, int qoff, int koff, i
   return hipGetLastError();
 }
 
+GRAG_API int grag_decay_attn_chunk() { return DECAY_CHUNK; }
+
+// ws: null (or max_q_len <= the chunk length) -> one workgroup per (sequence, head) walks the whole portion; else the
+// chunk-parallel passes over ws [nseq * ceil(max_q_len / chunk), H, d, vd] fp32.
 GRAG_API hipError_t grag_decay_attn_scan(const void* proj, int ld, int qoff, int koff, int voff, const float* decay,
                                          float* state, const int* slots, const int* q_start, const int* ctx_len,
-                                         float* out, int nseq, int H, int d, int vd, int nslots, int dt,
-                                         hipStream_t st) {
+                                         float* out, int nseq, int H, int d, int vd, int nslots, int dt, float* ws,
+                                         int max_q_len, hipStream_t st) {
   if (nseq <= 0) return hipSuccess;
   if (d > 256 || vd > 1024) return hipErrorInvalidValue;
-  DT_DISPATCH(dt, return launch_decay_scan<T>((const T*)proj, ld, qoff, koff, voff, decay, state, slots, q_start,
-                                              ctx_len, out, nseq, H, d, vd, nslots, st);)
+  if (ws == nullptr || max_q_len <= DECAY_CHUNK) {
+    DT_DISPATCH(dt, return (launch_decay_scan<T, 0>((const T*)proj, ld, qoff, koff, voff, decay, state, slots, q_start,
+                                                    ctx_len, out, nseq, H, d, vd, nslots, nullptr, 0, st));)
+  }
+  const int maxchunks = (max_q_len + DECAY_CHUNK - 1) / DECAY_CHUNK;
+  hipError_t e;
+  DT_DISPATCH(dt, e = (launch_decay_scan<T, 1>((const T*)proj, ld, qoff, koff, voff, decay, state, slots, q_start,
+                                               ctx_len, out, nseq, H, d, vd, nslots, ws, maxchunks, st));)
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL(decay_chunk_prefix_kernel, dim3(H, nseq), dim3(256), 0, st, decay, state, slots, q_start, ctx_len,
+                     ws, maxchunks, H, d, vd, nslots);
+  DT_DISPATCH(dt, e = (launch_decay_scan<T, 2>((const T*)proj, ld, qoff, koff, voff, decay, state, slots, q_start,
+                                               ctx_len, out, nseq, H, d, vd, nslots, ws, maxchunks, st));)
+  return e;
 }
 
 GRAG_API hipError_t grag_gated_rmsnorm(const float* x, const float* w, const void* proj, int ld, int goff, void* out,
@@ -582,14 +976,29 @@ GRAG_API hipError_t grag_gated_rmsnorm(const float* x, const float* w, const voi
   return hipGetLastError();
 }
 
+GRAG_API int grag_mingru_chunk() { return MINGRU_CHUNK; }
+
+// ws: null (or max_q_len <= the chunk length) -> one thread per channel walks the portion; else the two chunked
+// passes over ws [nseq * ceil(max_q_len / chunk), 2, W] fp32.
 GRAG_API hipError_t grag_mingru_scan(const void* proj, int ld, int zoff, int xoff, int goff, const float* bz,
                                      const float* bx, float* state, const int* slots, const int* q_start,
-                                     const int* ctx_len, void* out, int nseq, int W, int nslots, int dt,
-                                     hipStream_t st) {
+                                     const int* ctx_len, void* out, int nseq, int W, int nslots, int dt, float* ws,
+                                     int max_q_len, hipStream_t st) {
   if (nseq <= 0) return hipSuccess;
-  const dim3 grid((W + 255) / 256, nseq);
-  DT_DISPATCH(dt, hipLaunchKernelGGL(mingru_scan_kernel<T>, grid, dim3(256), 0, st, (const T*)proj, ld, zoff, xoff,
-                                     goff, bz, bx, state, slots, q_start, ctx_len, (T*)out, W, nslots);)
+  if (ws == nullptr || max_q_len <= MINGRU_CHUNK) {
+    const dim3 grid((W + 255) / 256, nseq);
+    DT_DISPATCH(dt, hipLaunchKernelGGL(mingru_scan_kernel<T>, grid, dim3(256), 0, st, (const T*)proj, ld, zoff, xoff,
+                                       goff, bz, bx, state, slots, q_start, ctx_len, (T*)out, W, nslots);)
+    return hipGetLastError();
+  }
+  const int maxchunks = (max_q_len + MINGRU_CHUNK - 1) / MINGRU_CHUNK;
+  const dim3 grid((W + 255) / 256, nseq, maxchunks);
+  DT_DISPATCH(dt, {
+    hipLaunchKernelGGL((mingru_chunk_kernel<T, 1>), grid, dim3(256), 0, st, (const T*)proj, ld, zoff, xoff, goff, bz,
+                       bx, state, slots, q_start, ctx_len, (T*)out, W, nslots, ws, maxchunks);
+    hipLaunchKernelGGL((mingru_chunk_kernel<T, 2>), grid, dim3(256), 0, st, (const T*)proj, ld, zoff, xoff, goff, bz,
+                       bx, state, slots, q_start, ctx_len, (T*)out, W, nslots, ws, maxchunks);
+  })
   return hipGetLastError();
 }
 

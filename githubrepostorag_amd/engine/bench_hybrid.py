@@ -1,0 +1,182 @@
+"""``bench.py --hybrid``: prefill and decode throughput of the Zofesun hybrid decoder beside the Qwen2 decoder of
+equal size (same width, heads, head size, FFN width, layer count, vocabulary; random weights, synthetic token
+ids), both through LLMEngine.generate, and a per-kernel table: each new kernel and the like kernel of Qwen2 as a
+fraction of the roofline of what bounds it (HBM bytes or matrix / vector flops)."""
+from __future__ import annotations
+
+import json
+import time
+
+import torch
+
+HBM_BPS = 8.0e12        # HBM3E
+MFMA_BF16 = 2.5e15      # dense bf16 matrix flop/s
+VALU_F32 = 1.57e14      # fp32 vector flop/s (fma = 2)
+
+SIZES = {
+    # name: (width, heads, kv_heads, head size, ffn, layers, mingru every)
+    "1b-like": (1536, 12, 2, 128, 8960, 8, 4),
+    "7b-like": (3584, 28, 4, 128, 18944, 4, 4),
+}
+VOCAB = 32768
+
+
+def _timed(fn, iters=10, warm=2):
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e-3 / iters
+
+
+def _models(name, dev):
+    from ..models.configs import DecoderConfig, zofesun_config
+    from ..models.qwen2 import Qwen2Model
+    from ..models.zofesun import ZofesunModel
+
+    W, H, G, D, ff, nl, every = SIZES[name]
+    zc = zofesun_config(f"zofesun-{name}", VOCAB, W, nl, heads=H, kv_heads=G, dim=D, vdim=D, lin_heads=H, lin_dim=D,
+                        lin_vdim=D, ff=ff, mingru_every=every)
+    qc = DecoderConfig(f"qwen2-{name}", VOCAB, W, ff, nl, H, G, D, max_position=32768)
+    return (lambda: ZofesunModel(zc, device=dev, seed=1)), (lambda: Qwen2Model(qc, device=dev, seed=1))
+
+
+def _engine_numbers(make, dev, batch, prompt_len, gen_len, graphs=True):
+    from .llm_engine import EngineConfig, LLMEngine
+    from .sequence import SamplingParams
+
+    model = make()
+    need = batch * (prompt_len + gen_len + 16)
+    eng = LLMEngine(model, None, EngineConfig(max_num_seqs=batch, max_model_len=prompt_len + gen_len + 16,
+                                              max_num_batched_tokens=max(8192, prompt_len), num_blocks=need // 16 + 2,
+                                              use_cuda_graph=graphs, enable_prefix_caching=False))
+    g = torch.Generator().manual_seed(0)
+    prompts = [torch.randint(0, VOCAB, (prompt_len,), generator=g).tolist() for _ in range(batch)]
+
+    def run(n):
+        t0 = time.perf_counter()
+        eng.generate(prompts, SamplingParams(max_tokens=n, temperature=0.0, ignore_eos=True))
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0
+
+    run(2)  # compile / capture
+    run(gen_len + 1)
+    t_pre = min(run(1) for _ in range(2))
+    t_all = min(run(gen_len + 1) for _ in range(2))
+    out = {"prefill_tok_s": round(batch * prompt_len / t_pre), "decode_tok_s": round(batch * gen_len / max(t_all - t_pre, 1e-9)),
+           "prefill_ms": round(t_pre * 1e3, 2), "decode_ms_per_step": round((t_all - t_pre) / gen_len * 1e3, 3)}
+    del eng, model
+    torch.cuda.empty_cache()
+    return out
+
+
+def _kernel_table(dev, H=28, G=4, D=128, W=3584, ff=18944, T=2048, B=64, ctx=2048, bs=16):
+    """[(kernel, seconds, bound, fraction of roofline)] for the new kernels and the like kernels of Qwen2."""
+    from ..ops.attention import AttnMetadata, paged_attention, sink_attention
+    from ..ops.elementwise import (clamped_glu, qkv_rope_kvstore, rope_cos_sin, rope_table, rope_vnorm_store, silu_mul)
+    from ..ops.norm import dyt_residual, rmsnorm
+    from ..ops.recurrent import decay_attention, gated_rmsnorm, mingru_scan
+
+    bf = torch.bfloat16
+    i32 = dict(dtype=torch.int32, device=dev)
+    rows = []
+
+    def add(name, sec, flops=0.0, bytes_=0.0, peak=MFMA_BF16):
+        t_c, t_m = flops / peak, bytes_ / HBM_BPS
+        bound = "flops" if t_c >= t_m else "bytes"
+        rows.append({"kernel": name, "us": round(sec * 1e6, 1), "bound": bound,
+                     "roofline_fraction": round(max(t_c, t_m) / sec, 4)})
+
+    # ---- prefill attention: one prompt of T tokens
+    nb = T // bs
+    kc = torch.randn(nb + 1, G, bs, D, device=dev).to(bf)
+    vc = torch.randn(nb + 1, G, bs, D, device=dev).to(bf)
+    q = torch.randn(T, H, D, device=dev).to(bf)
+    meta = AttnMetadata(q_start=torch.tensor([0, T], **i32), ctx_len=torch.tensor([T], **i32),
+                        block_tables=(torch.arange(nb, **i32) + 1).view(1, nb), slot_mapping=torch.arange(T, **i32) + bs,
+                        max_q_len=T, num_seqs=1, num_tokens=T, state_slots=torch.tensor([0], **i32))
+    sinks = torch.zeros(H, device=dev)
+    fl = 4.0 * T * T / 2 * H * D
+    add("sink_attn_prefill", _timed(lambda: sink_attention(q, kc, vc, meta, 0.09, sinks)), flops=fl)
+    add("qwen2 paged_attention prefill", _timed(lambda: paged_attention(q, kc, vc, meta, 0.09)), flops=fl)
+    # ---- decode attention: B rows of ctx keys
+    nbd = ctx // bs
+    kd = torch.randn(B * nbd + 1, G, bs, D, device=dev).to(bf)
+    vd_ = torch.randn(B * nbd + 1, G, bs, D, device=dev).to(bf)
+    qd = torch.randn(B, H, D, device=dev).to(bf)
+    part_o = torch.empty(8 * B * H * D, device=dev)
+    part_ml = torch.empty(8 * B * H * 2, device=dev)
+    dmeta = AttnMetadata(q_start=torch.arange(B + 1, **i32), ctx_len=torch.full((B,), ctx, **i32),
+                         block_tables=(torch.arange(B * nbd, **i32) + 1).view(B, nbd), slot_mapping=None, max_q_len=1,
+                         num_seqs=B, num_tokens=B, is_decode=True, num_splits=8, split_len=ctx // 8, part_o=part_o,
+                         part_ml=part_ml, state_slots=torch.arange(B, **i32))
+    by = 2.0 * B * ctx * G * D * 2
+    add("sink_attn_decode", _timed(lambda: sink_attention(qd, kd, vd_, dmeta, 0.09, sinks)), bytes_=by)
+    add("qwen2 paged_attention decode", _timed(lambda: paged_attention(qd, kd, vd_, dmeta, 0.09)), bytes_=by)
+    # ---- rotary + K/V store
+    proj = torch.randn(T, (H + 2 * G) * D, device=dev).to(bf)
+    pos = torch.arange(T, **i32)
+    tab = rope_table(T, D, 1e4, dev)
+    cs = rope_cos_sin(T, D, 1e4, dev)
+    by = T * (H + 2 * G) * D * 2 * 2.0
+    add("rope_vnorm_store", _timed(lambda: rope_vnorm_store(proj, 0, H * D, (H + G) * D, pos, tab, meta.slot_mapping, kc, vc,
+                                                            H, G, D, D, D, 1e-5)), bytes_=by)
+    add("qwen2 qkv_rope_kvstore", _timed(lambda: qkv_rope_kvstore(proj, None, pos, cs, meta.slot_mapping, kc, vc, H, G, D)),
+        bytes_=by)
+    # ---- norms at a sublayer boundary
+    resid = torch.randn(T, W, device=dev)
+    y = torch.randn(T, W, device=dev).to(bf)
+    w32, b32, wbf = torch.ones(W, device=dev), torch.zeros(W, device=dev), torch.ones(W, device=dev).to(bf)
+    add("dyt_residual (fp32 stream)", _timed(lambda: dyt_residual(resid, y, (0.5, w32, b32), pre=(0.5, w32, b32))),
+        bytes_=T * W * (2 + 4 + 4 + 2.0))
+    rb = torch.randn(T, W, device=dev).to(bf)
+    add("qwen2 add+rmsnorm (bf16 stream)", _timed(lambda: rmsnorm(y, wbf, 1e-6, residual=rb)), bytes_=T * W * 2 * 4.0)
+    # ---- GLU
+    gu = torch.randn(T, 2 * ff, device=dev).to(bf)
+    add("clamped_glu", _timed(lambda: clamped_glu(gu, 7.0)), bytes_=T * ff * 2 * 3.0)
+    add("qwen2 silu_mul", _timed(lambda: silu_mul(gu)), bytes_=T * ff * 2 * 3.0)
+    # ---- recurrent mixers (no like kernel in Qwen2; fp32 vector flops / state bytes)
+    pr = torch.randn(T, 4 * H * D, device=dev).to(bf)
+    dec = torch.full((H,), 0.99, device=dev)
+    S = torch.zeros(B + 1, H, D, D, device=dev)
+    add("decay_attn_scan prefill", _timed(lambda: decay_attention(pr, 0, H * D, 2 * H * D, dec, S, meta, H, D, D), 3, 1),
+        flops=4.0 * T * H * D * D, bytes_=T * 3 * H * D * 2.0, peak=VALU_F32)
+    prd = torch.randn(B, 4 * H * D, device=dev).to(bf)
+    add("decay_attn_scan decode", _timed(lambda: decay_attention(prd, 0, H * D, 2 * H * D, dec, S, dmeta, H, D, D)),
+        bytes_=2.0 * B * H * D * D * 4)
+    o = torch.randn(T, H * D, device=dev)
+    out = torch.empty(T, H * D, device=dev, dtype=bf)
+    add("gated_rmsnorm", _timed(lambda: gated_rmsnorm(o, w32[: H * D].contiguous(), pr, 3 * H * D, 1e-5, out)),
+        bytes_=T * H * D * (4 + 2 + 2.0))
+    gp = torch.randn(T, 3 * W, device=dev).to(bf)
+    Sg = torch.zeros(B + 1, W, device=dev)
+    add("mingru_scan prefill", _timed(lambda: mingru_scan(gp, 0, W, 2 * W, b32, b32, Sg, meta, W)), bytes_=T * W * 2 * 4.0)
+    gpd = torch.randn(B, 3 * W, device=dev).to(bf)
+    add("mingru_scan decode", _timed(lambda: mingru_scan(gpd, 0, W, 2 * W, b32, b32, Sg, dmeta, W)),
+        bytes_=B * W * (2 * 4 + 8.0))
+    return rows
+
+
+def run(args) -> dict:
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    sizes = {}
+    for name in SIZES:
+        mk_z, mk_q = _models(name, dev)
+        cell = {}
+        for batch, plen, glen in ((8, 2048, 64), (64, 1024, 64)):
+            key = f"B{batch}_P{plen}_G{glen}"
+            cell[key] = {"zofesun": _engine_numbers(mk_z, dev, batch, plen, glen),
+                         "qwen2": _engine_numbers(mk_q, dev, batch, plen, glen)}
+            print(json.dumps({"size": name, "shape": key, **cell[key]}), flush=True)
+        sizes[name] = cell
+    kernels = _kernel_table(dev)
+    for r in kernels:
+        print(json.dumps(r), flush=True)
+    return {"metric": "hybrid_vs_qwen2_tokens_per_s", "unit": "tokens/s", "dtype": "bf16", "data": "synthetic",
+            "sizes": sizes, "kernels": kernels}

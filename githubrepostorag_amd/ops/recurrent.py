@@ -10,8 +10,17 @@ from __future__ import annotations
 
 import torch
 
-from ._lib import call, ptr
+from ._lib import call, lib, ptr
 from .attention import AttnMetadata
+
+
+def _chunk_ws(kind: str, m: AttnMetadata, per_chunk: int, device) -> torch.Tensor | None:
+    """fp32 scratch for the chunk-parallel passes of a long portion ([sequences * chunks, per_chunk]); None when
+    every portion of the step fits one chunk (decode rows, short portions): the one-pass kernels take those."""
+    chunk = getattr(lib(), "grag_decay_attn_chunk" if kind == "decay" else "grag_mingru_chunk")()
+    if m.max_q_len <= chunk:
+        return None
+    return torch.empty(m.num_seqs * -(-m.max_q_len // chunk) * per_chunk, dtype=torch.float32, device=device)
 
 
 def _dt(t: torch.Tensor) -> int:
@@ -42,9 +51,10 @@ def decay_attention(proj: torch.Tensor, qoff: int, koff: int, voff: int, decay: 
             continue
         assert proj.stride(1) == 1 and state.dtype == torch.float32 and state.is_contiguous()
         x = proj[r0:r1]
+        ws = _chunk_ws("decay", m, H * d * vd, proj.device)
         call("grag_decay_attn_scan", ptr(x), proj.stride(0), qoff, koff, voff, ptr(decay), ptr(state),
              ptr(m.state_slots), ptr(m.q_start), ptr(m.ctx_len), ptr(out[r0:r1]), m.num_seqs, H, d, vd,
-             state.shape[0], _dt(proj))
+             state.shape[0], _dt(proj), ptr(ws), m.max_q_len)
     return out
 
 
@@ -96,9 +106,10 @@ def mingru_scan(proj: torch.Tensor, zoff: int, xoff: int, goff: int, bz: torch.T
             _mingru_cpu(proj[r0:r1].float(), zoff, xoff, goff, bz, bx, state, m, W, out[r0:r1])
             continue
         assert proj.stride(1) == 1 and state.dtype == torch.float32 and state.is_contiguous()
+        ws = _chunk_ws("mingru", m, 2 * W, proj.device)
         call("grag_mingru_scan", ptr(proj[r0:r1]), proj.stride(0), zoff, xoff, goff, ptr(bz), ptr(bx), ptr(state),
              ptr(m.state_slots), ptr(m.q_start), ptr(m.ctx_len), ptr(out[r0:r1]), m.num_seqs, W, state.shape[0],
-             _dt(proj))
+             _dt(proj), ptr(ws), m.max_q_len)
     return out
 
 

@@ -138,17 +138,17 @@ def _paged(k, v, bs, perm_seed=0, extra=3):
     return kc, vc, pages.to(torch.int32).view(1, nb), slots.to(torch.int32)
 
 
-def sink_attention_case(device, dtype, tol, T=150, far=(0, 15, 16, 17, 63, 64, 131), bs=16):
+def sink_attention_case(device, dtype, tol, T=150, far=(0, 15, 16, 17, 63, 64, 131), bs=16, d=12, vd=20):
     """One far key made to dominate (query and key scaled along one direction): the output is that key's value,
     wherever the key lies -- page borders, the first token -- for a prompt chunk and for a decoded token; the
     sink takes its share of the denominator."""
     from githubrepostorag_amd.ops.attention import AttnMetadata, sink_attention
 
-    H, G, d, vd = 4, 2, 12, 20
+    H, G = 4, 2
     g = torch.Generator().manual_seed(1)
     for key in far:
-        q = torch.randn(T, H, d, generator=g) * 0.3
-        k = torch.randn(T, G, d, generator=g) * 0.3
+        q = torch.randn(T, H, d, generator=g) * 0.3 * (12.0 / d) ** 0.5
+        k = torch.randn(T, G, d, generator=g) * 0.3 * (12.0 / d) ** 0.5
         v = torch.randn(T, G, vd, generator=g)
         k[key, :, 0] = 6.0
         q[T - 1, :, 0] = 6.0

@@ -32,6 +32,20 @@ def test_sink_attention_far_keys_and_page_borders(dtype, tol):
     T.sink_attention_case("cuda", dtype, tol, T=67, far=(0, 3, 4, 63, 64), bs=4)
 
 
+@pytest.mark.parametrize("d,vd", [(32, 48), (64, 16), (128, 128), (16, 256)])
+def test_sink_attention_matrix_core_shapes(d, vd):
+    """bf16 with head sizes in multiples of 16: prompt portions of >= 16 queries run on the matrix cores."""
+    T.sink_attention_case("cuda", torch.bfloat16, 0.03, T=150, far=(0, 15, 16, 64, 131), d=d, vd=vd)
+    T.sink_attention_case("cuda", torch.bfloat16, 0.03, T=200, far=(63, 128, 191), bs=4, d=d, vd=vd)
+
+
+def test_matrix_core_shapes_through_the_engine():
+    kw = dict(dim=32, vdim=48, rot_dims=16, lin_dim=16, lin_vdim=32)
+    C.case_whole_and_layers("cuda", BF16, torch.bfloat16, **kw)
+    C.case_prefill_vs_decode("cuda", BF16, torch.bfloat16, n=150, **kw)
+    C.case_prefill_vs_decode("cuda", F32, torch.float32, n=150, **kw)
+
+
 def test_sink_attention_wide_heads():
     """Head sizes past one 64-lane pass, and a key tile that does not fit 64 keys."""
     from githubrepostorag_amd.ops.attention import AttnMetadata, sink_attention

@@ -75,8 +75,8 @@ def case_whole_and_layers(device, tol, dtype=torch.float32, **cfg_kw):
         assert err < tol, (r, err)
 
 
-def case_prefill_vs_decode(device, tol, dtype=torch.float32, n=70):
-    cfg = O.make_config()
+def case_prefill_vs_decode(device, tol, dtype=torch.float32, n=70, **cfg_kw):
+    cfg = O.make_config(**cfg_kw)
     sd = O.make_weights(cfg, seed=5)
     toks = tokens(cfg, n, 1)
     want, _ = O.forward(cfg, sd, toks)
