@@ -245,7 +245,7 @@ sink_attn_prefill_kernel(const T* __restrict__ q, const T* __restrict__ k_cache,
 //   O^T += V^T P^T   with the fp32 weights split into bf16 hi + lo parts (two products): 16 mantissa bits of P
 //                    reach the accumulator, below the bf16 rounding of V and of the stored output.
 template <int NKM, int NVM>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256, 3)
 sink_attn_prefill_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_cache,
                               const bf16* __restrict__ v_cache, bf16* __restrict__ out, int out_ld,
                               const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ q_start,
@@ -383,6 +383,195 @@ sink_attn_prefill_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict
         *reinterpret_cast<bf16x4_t*>(orow + 16 * v + 4 * quad) = o;
       }
     }
+  }
+}
+
+// decode on the matrix cores (bf16, d and vd multiples of 16, H / G <= 16): grid (key splits, G, nseq), 4 waves.
+// The 16 fragment columns are the query heads that share one kv head (GQA packing: K / V are read once for all of
+// them).  The block stages 64-key tiles as the prefill kernel does; wave w owns keys 16w .. 16w+15 of every tile with
+// its own running (max, sum, O^T) and the four waves merge through LDS at the end.  With nsplit > 1 every split
+// writes its unnormalised O and (max, sum) to part_o [nsplit, nseq, H, vd] / part_ml [nsplit, nseq, H, 2] and
+// sink_attn_combine_kernel merges them; the sink term enters once (split 0, wave 0).
+template <int NKM, int NVM>
+__global__ void __launch_bounds__(256, 3)
+sink_attn_decode_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_cache,
+                             const bf16* __restrict__ v_cache, bf16* __restrict__ out, int out_ld,
+                             const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ ctx_len,
+                             const float* __restrict__ sinks, int H, int G, int d, int vd, int BS, float scale,
+                             float out_scale, int nblocks, int nsplit, int split_len, float* __restrict__ part_o,
+                             float* __restrict__ part_ml) {
+  constexpr int KT = 64;
+  extern __shared__ __attribute__((aligned(16))) char smem_raw[];
+  const int sp = blockIdx.x, g = blockIdx.y, seq = blockIdx.z, nseq = gridDim.z;
+  const int R = H / G;
+  const int ctx = ctx_len[seq];
+  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+  const int ql = lane & 15, quad = lane >> 4;
+  const int nk = d >> 4, nv = vd >> 4;
+  const int kstride = d + 8, vstride = KT + 4;
+  short* Ks = reinterpret_cast<short*>(smem_raw);
+  short* Vt = Ks + KT * kstride;
+  const bool col_ok = ql < R;
+  const int head = g * R + (col_ok ? ql : 0);
+  bf16x4_t qf[NKM];
+#pragma unroll
+  for (int ks = 0; ks < NKM; ++ks) {
+    qf[ks] = bf16x4_t{0, 0, 0, 0};
+    if (ks < nk && col_ok)
+      qf[ks] = *reinterpret_cast<const bf16x4_t*>(q + ((size_t)seq * H + head) * d + ks * 16 + quad * 4);
+  }
+  const bool has_sink = sp == 0 && wid == 0;
+  float m = has_sink ? sinks[head] : -INFINITY, l = has_sink ? 1.f : 0.f;
+  f32x4_t acc[NVM];
+#pragma unroll
+  for (int v = 0; v < NVM; ++v) acc[v] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  const int kbeg = nsplit > 1 ? sp * split_len : 0;
+  const int kend = nsplit > 1 ? min(ctx, kbeg + split_len) : ctx;
+  const int* bt = block_tables + (size_t)seq * bt_stride;
+  const int dv8 = d >> 3, vv8 = vd >> 3;
+  for (int k0 = kbeg; k0 < kend; k0 += KT) {
+    __syncthreads();
+    const int kn = min(KT, kend - k0);
+    for (int idx = threadIdx.x; idx < KT * dv8; idx += 256) {
+      const int kk = idx / dv8, c = idx - kk * dv8;
+      bf16x8_t v = bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
+      if (kk < kn) {
+        const int key = k0 + kk;
+        const int blk = bt[key / BS];
+        if (index_ok(blk, nblocks, ERR_BLOCK_DECODE))
+          v = *reinterpret_cast<const bf16x8_t*>(k_cache + (((size_t)blk * G + g) * BS + key % BS) * d + c * 8);
+      }
+      *reinterpret_cast<bf16x8_t*>(Ks + kk * kstride + c * 8) = v;
+    }
+    for (int idx = threadIdx.x; idx < KT * vv8; idx += 256) {
+      const int kk = idx / vv8, c = idx - kk * vv8;
+      bf16x8_t v = bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
+      if (kk < kn) {
+        const int key = k0 + kk;
+        const int blk = bt[key / BS];
+        if (blk >= 0 && blk < nblocks)
+          v = *reinterpret_cast<const bf16x8_t*>(v_cache + (((size_t)blk * G + g) * BS + key % BS) * vd + c * 8);
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) Vt[(c * 8 + e) * vstride + kk] = v[e];
+    }
+    __syncthreads();
+    if (16 * wid >= kn) continue;  // this wave's 16 keys lie past the split's end
+    f32x4_t st = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < NKM; ++ks) {
+      if (ks < nk) {
+        const bf16x4_t a = *reinterpret_cast<const bf16x4_t*>(Ks + (16 * wid + ql) * kstride + ks * 16 + quad * 4);
+        st = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, qf[ks], st, 0, 0, 0);
+      }
+    }
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const bool vis = col_ok && 16 * wid + 4 * quad + i < kn;
+      st[i] = vis ? st[i] * scale : -INFINITY;
+      tmax = fmaxf(tmax, st[i]);
+    }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    const float mn = fmaxf(m, tmax);
+    const float alpha = m == -INFINITY ? 0.f : expf(m - mn);
+    float psum = 0.f;
+    bf16x4_t ph, pl;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float p = st[i] == -INFINITY ? 0.f : expf(st[i] - mn);
+      psum += p;
+      const short hi = f2bits(p);
+      ph[i] = hi;
+      pl[i] = f2bits(p - bits2f(hi));
+    }
+    psum += __shfl_xor(psum, 16, 64);
+    psum += __shfl_xor(psum, 32, 64);
+    l = l * alpha + psum;
+    m = mn;
+#pragma unroll
+    for (int v = 0; v < NVM; ++v) {
+      if (v < nv) {
+        const bf16x4_t a = *reinterpret_cast<const bf16x4_t*>(Vt + (16 * v + ql) * vstride + 16 * wid + 4 * quad);
+        acc[v] *= alpha;
+        acc[v] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, ph, acc[v], 0, 0, 0);
+        acc[v] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, pl, acc[v], 0, 0, 0);
+      }
+    }
+  }
+  // merge the four waves: (m, l) per column, O^T [vd][16 columns] per wave
+  __syncthreads();
+  float* Mw = reinterpret_cast<float*>(smem_raw);  // [4][16]
+  float* Lw = Mw + 64;                             // [4][16]
+  float* Aw = Lw + 64;                             // [4][vd][16]
+  if (quad == 0) {
+    Mw[wid * 16 + ql] = m;
+    Lw[wid * 16 + ql] = l;
+  }
+#pragma unroll
+  for (int v = 0; v < NVM; ++v)
+    if (v < nv)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) Aw[((size_t)wid * vd + 16 * v + 4 * quad + i) * 16 + ql] = acc[v][i];
+  __syncthreads();
+  float M = -INFINITY;
+  for (int w = 0; w < 4; ++w) M = fmaxf(M, Mw[w * 16 + ql]);
+  float f[4], L = 0.f;
+  for (int w = 0; w < 4; ++w) {
+    const float mw = Mw[w * 16 + ql];
+    f[w] = mw == -INFINITY ? 0.f : expf(mw - M);
+    L += Lw[w * 16 + ql] * f[w];
+  }
+  if (!col_ok) return;
+#pragma unroll
+  for (int v = 0; v < NVM; ++v) {
+    if (v < nv && (v & 3) == wid) {
+      f32x4_t o;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float x = 0.f;
+        for (int w = 0; w < 4; ++w) x = fmaf(Aw[((size_t)w * vd + 16 * v + 4 * quad + i) * 16 + ql], f[w], x);
+        o[i] = x;
+      }
+      if (nsplit > 1) {
+        *reinterpret_cast<f32x4_t*>(part_o + (((size_t)sp * nseq + seq) * H + head) * vd + 16 * v + 4 * quad) = o;
+      } else {
+        const float r = out_scale / L;
+        bf16x4_t ob;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) ob[i] = f2bits(o[i] * r);
+        *reinterpret_cast<bf16x4_t*>(out + (size_t)seq * out_ld + head * vd + 16 * v + 4 * quad) = ob;
+      }
+    }
+  }
+  if (nsplit > 1 && wid == 0 && quad == 0) {
+    float* ml = part_ml + (((size_t)sp * nseq + seq) * H + head) * 2;
+    ml[0] = M;
+    ml[1] = L;
+  }
+}
+
+// out = out_scale * sum_s O_s e^(m_s - M) / sum_s l_s e^(m_s - M) over the key splits; grid (H, nseq).
+__global__ void sink_attn_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                         bf16* __restrict__ out, int out_ld, int nsplit, int nseq, int H, int vd,
+                                         float out_scale) {
+  const int h = blockIdx.x, seq = blockIdx.y;
+  float M = -INFINITY;
+  for (int s = 0; s < nsplit; ++s) M = fmaxf(M, part_ml[(((size_t)s * nseq + seq) * H + h) * 2]);
+  float L = 0.f;
+  for (int s = 0; s < nsplit; ++s) {
+    const float* ml = part_ml + (((size_t)s * nseq + seq) * H + h) * 2;
+    L += ml[0] == -INFINITY ? 0.f : ml[1] * expf(ml[0] - M);
+  }
+  const float r = out_scale / L;
+  for (int j = threadIdx.x; j < vd; j += blockDim.x) {
+    float o = 0.f;
+    for (int s = 0; s < nsplit; ++s) {
+      const float ms = part_ml[(((size_t)s * nseq + seq) * H + h) * 2];
+      if (ms != -INFINITY) o = fmaf(part_o[(((size_t)s * nseq + seq) * H + h) * vd + j], expf(ms - M), o);
+    }
+    out[(size_t)seq * out_ld + h * vd + j] = (bf16)(o * r);
   }
 }
 
@@ -597,13 +786,15 @@ sink_attn_decode_kernel(const T* __restrict__ q, const T* __restrict__ k_cache, 
 constexpr int DECAY_CHUNK = 64;
 
 template <typename T, int DMAX, int MODE>
-__global__ void decay_attn_scan_kernel(const T* __restrict__ proj, int ld, int qoff, int koff, int voff,
+__global__ void __launch_bounds__(256)
+decay_attn_scan_kernel(const T* __restrict__ proj, int ld, int qoff, int koff, int voff,
                                        const float* __restrict__ decay, float* __restrict__ state,
                                        const int* __restrict__ slots, const int* __restrict__ q_start,
                                        const int* __restrict__ ctx_len, float* __restrict__ out, int H, int d, int vd,
                                        int nslots, float* __restrict__ ws, int maxchunks) {
   constexpr int TB = 16;
-  extern __shared__ float smem[];  // [TB][2][d]
+  extern __shared__ __attribute__((aligned(16))) float smem[];  // [TB][2][dp], dp = d rounded up to 4 (16-B rows)
+  const int dp = (d + 3) & ~3;
   const int seq = blockIdx.y, h = blockIdx.x;
   int qa = q_start[seq], qlen = q_start[seq + 1] - qa;
   if (qlen <= 0) return;
@@ -634,21 +825,29 @@ __global__ void decay_attn_scan_kernel(const T* __restrict__ proj, int ld, int q
       const int tt = idx / (2 * d), r = idx - tt * 2 * d;
       const int which = r / d, i = r - which * d;
       const T* row = proj + (size_t)(qa + t0 + tt) * ld + (which ? koff : qoff) + h * d;
-      smem[idx] = silu_acc(ldf(row + i));
+      smem[(tt * 2 + which) * dp + i] = silu_acc(ldf(row + i));
     }
     __syncthreads();
     if (j < vd) {
       for (int tt = 0; tt < nb; ++tt) {
         const size_t tok = (size_t)(qa + t0 + tt);
         const float vj = silu_acc(ldf(proj + tok * ld + voff + h * vd + j));
-        const float* qs = smem + tt * 2 * d;
-        const float* ks = qs + d;
+        const f32x4_t* qs = reinterpret_cast<const f32x4_t*>(smem + tt * 2 * dp);
+        const f32x4_t* ks = reinterpret_cast<const f32x4_t*>(smem + (tt * 2 + 1) * dp);
         float o = 0.f;
 #pragma unroll
-        for (int i = 0; i < DMAX; ++i) {
-          if (i < d) {
-            S[i] = fmaf(lam, S[i], ks[i] * vj);
-            if (MODE != 1) o = fmaf(S[i], qs[i], o);
+        for (int i4 = 0; i4 < DMAX / 4; ++i4) {
+          if (i4 * 4 < d) {  // (rows are zero-free past d only up to dp: the i < d tests below keep them out)
+            const f32x4_t k4 = ks[i4];
+            const f32x4_t q4 = MODE != 1 ? qs[i4] : f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const int i = i4 * 4 + e;
+              if (i < d) {
+                S[i] = fmaf(lam, S[i], k4[e] * vj);
+                if (MODE != 1) o = fmaf(S[i], q4[e], o);
+              }
+            }
           }
         }
         if (MODE != 1) out[tok * (size_t)(H * vd) + h * vd + j] = o;
@@ -897,12 +1096,46 @@ GRAG_API hipError_t grag_sink_attn_prefill(const void* q, const void* k_cache, c
   return hipGetLastError();
 }
 
+// part_o / part_ml: fp32 scratch of nsplit * nseq * H * (vd | 2) floats for nsplit > 1 key splits of split_len keys
+// (a multiple of 64); the split plan is taken by the matrix-core kernel only -- the other kernels walk all keys.
 GRAG_API hipError_t grag_sink_attn_decode(const void* q, const void* k_cache, const void* v_cache, void* out,
                                           int out_ld, const int* block_tables, int bt_stride, const int* ctx_len,
                                           const float* sinks, int nseq, int H, int G, int d, int vd, int BS,
-                                          float scale, float out_scale, int nblocks, int dt, hipStream_t st) {
+                                          float scale, float out_scale, int nblocks, int dt, int nsplit,
+                                          int split_len, float* part_o, float* part_ml, hipStream_t st) {
   if (nseq <= 0) return hipSuccess;
   if (vd > 64 * SA_VC || G <= 0 || H % G) return hipErrorInvalidValue;
+  if (dt == 0 && d % 16 == 0 && vd % 16 == 0 && d <= 256 && vd <= 256 && H / G <= 16 && out_ld % 4 == 0 &&
+      (reinterpret_cast<uintptr_t>(out) & 7) == 0 && (reinterpret_cast<uintptr_t>(q) & 7) == 0 && nseq <= 65535) {
+    if (nsplit < 1 || part_o == nullptr || part_ml == nullptr || split_len % 64) nsplit = 1;
+    const size_t kvb = ((size_t)64 * (d + 8) + (size_t)vd * (64 + 4)) * sizeof(short);
+    const size_t mgb = (128 + (size_t)4 * vd * 16) * sizeof(float);
+    const size_t mb = kvb > mgb ? kvb : mgb;
+    const dim3 mgrid(nsplit, G, nseq);
+#define SD_MFMA(NK, NV)                                                                                              \
+  {                                                                                                                  \
+    if (mb > 48 * 1024) {                                                                                            \
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&sink_attn_decode_mfma_kernel<NK, NV>),       \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)mb);                       \
+      if (e != hipSuccess) return e;                                                                                 \
+    }                                                                                                                \
+    hipLaunchKernelGGL((sink_attn_decode_mfma_kernel<NK, NV>), mgrid, dim3(256), mb, st, (const bf16*)q,             \
+                       (const bf16*)k_cache, (const bf16*)v_cache, (bf16*)out, out_ld, block_tables, bt_stride,      \
+                       ctx_len, sinks, H, G, d, vd, BS, scale, out_scale, nblocks, nsplit, split_len, part_o,        \
+                       part_ml);                                                                                     \
+  }
+    const int nk = d / 16, nv = vd / 16;
+    if (nk <= 4 && nv <= 4) SD_MFMA(4, 4)
+    else if (nk <= 8 && nv <= 8) SD_MFMA(8, 8)
+    else if (nk <= 8) SD_MFMA(8, 16)
+    else if (nv <= 8) SD_MFMA(16, 8)
+    else SD_MFMA(16, 16)
+#undef SD_MFMA
+    if (nsplit > 1)
+      hipLaunchKernelGGL(sink_attn_combine_kernel, dim3(H, nseq), dim3(vd <= 64 ? 64 : 128), 0, st, part_o, part_ml,
+                         (bf16*)out, out_ld, nsplit, nseq, H, vd, out_scale);
+    return hipGetLastError();
+  }
   const size_t bytes = ((size_t)d + 4 * 64 + 8 + 4 * (size_t)vd) * sizeof(float);
   if (dt == 0 && d % 8 == 0 && vd % 2 == 0 && vd <= 256) {
     hipLaunchKernelGGL(sink_attn_decode_vec_kernel, dim3(H, nseq), dim3(256), bytes, st, (const bf16*)q,
@@ -922,7 +1155,7 @@ static hipError_t launch_decay_scan(const T* proj, int ld, int qoff, int koff, i
                                     int nseq, int H, int d, int vd, int nslots, float* ws, int maxchunks,
                                     hipStream_t st) {
   const int threads = ((vd + 63) / 64) * 64;
-  const size_t bytes = (size_t)16 * 2 * d * sizeof(float);
+  const size_t bytes = (size_t)16 * 2 * ((d + 3) & ~3) * sizeof(float);
   const dim3 grid(H, nseq, MODE == 0 ? 1 : maxchunks);
 #define DECAY_LAUNCH(DM)                                                                                     \
   hipLaunchKernelGGL((decay_attn_scan_kernel<T, DM, MODE>), grid, dim3(threads), bytes, st, proj, ld, qoff, koff, \
@@ -951,7 +1184,7 @@ GRAG_API hipError_t grag_decay_attn_scan(const void* proj, int ld, int qoff, int
                                          float* out, int nseq, int H, int d, int vd, int nslots, int dt, float* ws,
                                          int max_q_len, hipStream_t st) {
   if (nseq <= 0) return hipSuccess;
-  if (d > 256 || vd > 1024) return hipErrorInvalidValue;
+  if (d > 256 || vd > 256) return hipErrorInvalidValue;
   if (ws == nullptr || max_q_len <= DECAY_CHUNK) {
     DT_DISPATCH(dt, return (launch_decay_scan<T, 0>((const T*)proj, ld, qoff, koff, voff, decay, state, slots, q_start,
                                                     ctx_len, out, nseq, H, d, vd, nslots, nullptr, 0, st));)

@@ -102,8 +102,12 @@ class ZofesunModel:
         self.tp = tp or Group([0])
         if not self.tp.trivial:
             raise NotImplementedError("the hybrid decoder runs on one GPU per replica (no tensor parallelism)")
-        # the engine sizes its split-KV scratch from these (this model's decode attention merges in-launch)
-        self.hq = self.hkv = self.head_dim = 1
+        # the engine sizes the decode attention's split-KV scratch (hq * head_dim floats per row and split) and
+        # picks its split plan (hkv) from these: the widest attention among the layers
+        att = [L.mixer.left for L in cfg.layers if L.mixer.kind == "parallel"]
+        self.hq = max([a.heads for a in att], default=1)
+        self.hkv = min([a.kv_heads for a in att], default=1)
+        self.head_dim = max([a.vdim for a in att], default=1)
         self.runs = cfg.layer_runs()
         self._tables: dict = {}
         self._max_pos = 0

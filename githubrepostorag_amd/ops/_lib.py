@@ -83,7 +83,7 @@ _SIGS = {
     "grag_dyt_residual": [P, F, P, P, P, P, P, F, P, P, P, I, I, I, P],
     "grag_rope_vnorm_store": [P, I, I, I, I, P, P, I, P, P, P, P, I, I, I, I, I, I, I, ctypes.c_long, F, I, P],
     "grag_sink_attn_prefill": [P, P, P, P, I, P, I, P, P, P, I, I, I, I, I, I, I, F, F, I, I, P],
-    "grag_sink_attn_decode": [P, P, P, P, I, P, I, P, P, I, I, I, I, I, I, F, F, I, I, P],
+    "grag_sink_attn_decode": [P, P, P, P, I, P, I, P, P, I, I, I, I, I, I, F, F, I, I, I, I, P, P, P],
     "grag_decay_attn_scan": [P, I, I, I, I, P, P, P, P, P, P, I, I, I, I, I, I, P, I, P],
     "grag_decay_attn_chunk": [],
     "grag_mingru_chunk": [],

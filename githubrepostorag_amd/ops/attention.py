@@ -464,9 +464,16 @@ def sink_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
     assert q.is_contiguous() and out.stride(1) == 1 and sinks.dtype == torch.float32
     dt = 0 if q.dtype == torch.bfloat16 else 1
     if meta.is_decode and meta.max_q_len == 1:
+        # key splits (flash-decoding) when the step brings a plan and scratch that holds it
+        nsplit = meta.num_splits
+        if (nsplit > 1 and (meta.part_o is None or meta.part_ml is None
+                            or meta.part_o.numel() < nsplit * meta.num_seqs * H * vd
+                            or meta.part_ml.numel() < nsplit * meta.num_seqs * H * 2)):
+            nsplit = 1
         call("grag_sink_attn_decode", ptr(q), ptr(k_cache), ptr(v_cache), ptr(out), out.stride(0),
              ptr(meta.block_tables), meta.block_tables.stride(0), ptr(meta.ctx_len), ptr(sinks), meta.num_seqs, H, G,
-             d, vd, BS, float(scale), float(out_scale), k_cache.shape[0], dt)
+             d, vd, BS, float(scale), float(out_scale), k_cache.shape[0], dt, nsplit, meta.split_len if nsplit > 1 else 0,
+             ptr(meta.part_o) if nsplit > 1 else None, ptr(meta.part_ml) if nsplit > 1 else None)
     else:
         call("grag_sink_attn_prefill", ptr(q), ptr(k_cache), ptr(v_cache), ptr(out), out.stride(0),
              ptr(meta.block_tables), meta.block_tables.stride(0), ptr(meta.q_start), ptr(meta.ctx_len), ptr(sinks),

@@ -39,11 +39,58 @@ def test_sink_attention_matrix_core_shapes(d, vd):
     T.sink_attention_case("cuda", torch.bfloat16, 0.03, T=200, far=(63, 128, 191), bs=4, d=d, vd=vd)
 
 
+@pytest.mark.parametrize("H,G,d,vd", [(4, 2, 32, 48), (14, 2, 128, 128), (16, 1, 16, 32), (3, 3, 64, 16)])
+def test_decode_key_splits(H, G, d, vd):
+    """One decoded token over a long context cut into key splits that are merged afterwards: the sink counts once,
+    empty splits (a context shorter than the plan) add nothing, heads that share a kv head ride in one block."""
+    from githubrepostorag_amd.ops.attention import AttnMetadata, sink_attention
+    import zofesun_oracle as O
+
+    g = torch.Generator().manual_seed(5)
+    bf = torch.bfloat16
+    lens = [700, 65, 1, 256]
+    B, bs = len(lens), 16
+    i32 = dict(dtype=torch.int32, device="cuda")
+    nbmax = -(-max(lens) // bs)
+    kc = torch.zeros(B * nbmax + 1, G, bs, d, dtype=bf, device="cuda")
+    vc = torch.zeros(B * nbmax + 1, G, bs, vd, dtype=bf, device="cuda")
+    bt = torch.zeros(B, nbmax, dtype=torch.int32)
+    sinks = torch.randn(H, generator=g)
+    qs, want = [], []
+    perm = torch.randperm(B * nbmax, generator=g) + 1
+    for b, n in enumerate(lens):
+        q = (torch.randn(n, H, d, generator=g) * 0.4).to(bf).float()
+        k = (torch.randn(n, G, d, generator=g) * 0.4).to(bf).float()
+        v = torch.randn(n, G, vd, generator=g).to(bf).float()
+        k[n // 3, :, 1] = 5.0
+        q[n - 1, :, 1] = 4.0  # a key far back that stands out
+        want.append(O.sink_attention(q[n - 1:].double(), k.double(), v.double(), 0.7, sinks.double())[0]
+                    if n == 1 else O.sink_attention(q.double(), k.double(), v.double(), 0.7, sinks.double())[n - 1])
+        pages = perm[b * nbmax:(b + 1) * nbmax]
+        bt[b] = pages.to(torch.int32)
+        pos = torch.arange(n)
+        kc[pages[pos // bs], :, pos % bs] = k.to(bf).cuda()
+        vc[pages[pos // bs], :, pos % bs] = v.to(bf).cuda()
+        qs.append(q[n - 1])
+    qd = torch.stack(qs).to(bf).cuda().contiguous()
+    for nsplit, split_len in ((1, 1 << 30), (4, 256), (16, 64), (8, 128)):
+        meta = AttnMetadata(q_start=torch.arange(B + 1, **i32), ctx_len=torch.tensor(lens, **i32),
+                            block_tables=bt.cuda(), slot_mapping=None, max_q_len=1, num_seqs=B, num_tokens=B,
+                            is_decode=True, num_splits=nsplit, split_len=split_len,
+                            part_o=torch.full((nsplit * B * H * vd,), float("nan"), device="cuda"),
+                            part_ml=torch.full((nsplit * B * H * 2,), float("nan"), device="cuda"))
+        got = sink_attention(qd, kc, vc, meta, 0.7, sinks.cuda(), out_scale=1.5).double().cpu().view(B, H, vd)
+        for b in range(B):
+            err = float((got[b] - 1.5 * want[b]).abs().max())
+            assert err < 0.03, (nsplit, b, err)
+
+
 def test_matrix_core_shapes_through_the_engine():
     kw = dict(dim=32, vdim=48, rot_dims=16, lin_dim=16, lin_vdim=32)
     C.case_whole_and_layers("cuda", BF16, torch.bfloat16, **kw)
     C.case_prefill_vs_decode("cuda", BF16, torch.bfloat16, n=150, **kw)
     C.case_prefill_vs_decode("cuda", F32, torch.float32, n=150, **kw)
+    C.case_generate("cuda", torch.bfloat16, graphs=True, window=4, tol=0.05, **kw)
 
 
 def test_sink_attention_wide_heads():
