@@ -47,8 +47,13 @@ __global__ void dyt_residual_kernel(const T* __restrict__ y, float a1, const flo
                                     const float* __restrict__ add_rows, const float* __restrict__ add_vec, float a2,
                                     const float* __restrict__ w2, const float* __restrict__ b2, T* __restrict__ out,
                                     int H) {
+  // grid (T, ceil(H / 1024)): 256 threads x 4 strided elements, so a few decode rows still spread over the chip
   const size_t base = (size_t)blockIdx.x * H;
-  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+  const int i0 = blockIdx.y * 1024 + threadIdx.x;
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const int i = i0 + k * 256;
+    if (i >= H) break;
     float x = resid[base + i];
     if (y != nullptr) x += tanhf(a1 * ldf(y + base + i)) * w1[i] + b1[i];
     if (add_rows != nullptr) x += add_rows[base + i];
@@ -62,45 +67,20 @@ __global__ void dyt_residual_kernel(const T* __restrict__ y, float a1, const flo
 // proj [T, ld]: q heads at column qoff (H x d), k heads at koff (G x d), v heads at voff (G x vd).
 // q_out [T, H*d] = rotated q; k_cache [nblk, G, BS, d] <- rotated k; v_cache [nblk, G, BS, vd] <- v / rms(v).
 // Rotation: the first rd dims of a head, dim i paired with i + rd/2; table row p = cos[0:rd/2] | sin[0:rd/2] (fp32).
+// grid (T, H + G + G): one wave per (token, head): q heads, then k heads, then v heads.
 template <typename T>
 __global__ void rope_vnorm_store_kernel(const T* __restrict__ proj, int ld, int qoff, int koff, int voff,
                                         const int* __restrict__ positions, const float* __restrict__ table,
                                         int table_rows, const int* __restrict__ slot_mapping, T* __restrict__ q_out,
                                         T* __restrict__ k_cache, T* __restrict__ v_cache, int H, int G, int d, int vd,
                                         int rd, int BS, long nslots, float eps) {
-  const int t = blockIdx.x;
+  const int t = blockIdx.x, hb = blockIdx.y, lane = threadIdx.x;
   const T* row = proj + (size_t)t * ld;
-  const int pos = positions[t];
-  const bool pos_ok = rd == 0 || index_ok(pos, table_rows, ERR_ROPE_POS);
-  const float* cs = table + (size_t)(pos_ok ? pos : 0) * rd;
-  const int half = rd >> 1;
   const int slot = slot_mapping[t];
   const bool store = slot >= 0 && index_ok(slot, nslots, ERR_KV_SLOT);
   const int blk = store ? slot / BS : 0, off = store ? slot % BS : 0;
-  const int nq = H * d, nk = G * d;
-  for (int e = threadIdx.x; e < nq + nk; e += blockDim.x) {
-    const bool isq = e < nq;
-    const int f = isq ? e : e - nq;
-    const int hh = f / d, i = f - hh * d;
-    const T* x = row + (isq ? qoff : koff) + hh * d;
-    float v = ldf(x + i);
-    if (i < rd && pos_ok) {
-      if (i < half) {
-        v = v * cs[i] - ldf(x + i + half) * cs[half + i];
-      } else {
-        const int j = i - half;
-        v = v * cs[j] + ldf(x + j) * cs[half + j];
-      }
-    }
-    if (isq) {
-      stf(q_out + (size_t)t * nq + e, v);
-    } else if (store) {
-      stf(k_cache + (((size_t)blk * G + hh) * BS + off) * d + i, v);
-    }
-  }
-  // values: one wave per kv head, RMS over vd in fp32
-  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6, nw = blockDim.x >> 6;
-  for (int g = wid; g < G; g += nw) {
+  if (hb >= H + G) {  // a value head: RMS over vd in fp32
+    const int g = hb - H - G;
     const T* x = row + voff + g * vd;
     float ss = 0.f;
     for (int i = lane; i < vd; i += 64) {
@@ -111,6 +91,28 @@ __global__ void rope_vnorm_store_kernel(const T* __restrict__ proj, int ld, int 
     const float r = 1.f / sqrtf(ss / (float)vd + eps);
     if (store)
       for (int i = lane; i < vd; i += 64) stf(v_cache + (((size_t)blk * G + g) * BS + off) * vd + i, ldf(x + i) * r);
+    return;
+  }
+  const int pos = positions[t];
+  const bool pos_ok = rd == 0 || index_ok(pos, table_rows, ERR_ROPE_POS);
+  const float* cs = table + (size_t)(pos_ok ? pos : 0) * rd;
+  const int half = rd >> 1;
+  const bool isq = hb < H;
+  const int hh = isq ? hb : hb - H;
+  const T* x = row + (isq ? qoff : koff) + hh * d;
+  if (!isq && !store) return;
+  T* dst = isq ? q_out + ((size_t)t * H + hh) * d : k_cache + (((size_t)blk * G + hh) * BS + off) * d;
+  for (int i = lane; i < d; i += 64) {
+    float v = ldf(x + i);
+    if (i < rd && pos_ok) {
+      if (i < half) {
+        v = v * cs[i] - ldf(x + i + half) * cs[half + i];
+      } else {
+        const int j = i - half;
+        v = v * cs[j] + ldf(x + j) * cs[half + j];
+      }
+    }
+    stf(dst + i, v);
   }
 }
 
@@ -238,12 +240,14 @@ sink_attn_prefill_kernel(const T* __restrict__ q, const T* __restrict__ k_cache,
 }
 
 // prefill on the matrix cores (bf16 activations, d and vd multiples of 16): grid (tiles of 64 queries, H, nseq), 4 waves
-// of 16 queries.  Per 64-key tile (K [64][d+8] and V^T [vd][64+4] staged in LDS as bf16):
+// of 16 queries.  Per 64-key tile (K [64][d+8] and V [64][vd+8] staged in LDS as bf16, both row-major):
 //   S^T = K Q^T      v_mfma_f32_16x16x16_bf16: bf16 products are exact in fp32, fp32 accumulation; the C fragment
-//                    (rows = keys 4*(lane/16)+i, column = query lane%16) is the B fragment of the next product,
+//                    (rows = keys 4*(lane/16)+i, column = query lane%16) is, read as "row = query lane%16, k = keys
+//                    4*(lane/16)+i", exactly the A fragment of the next product: P never leaves the registers,
 //   softmax in fp32  per query = per lane column: max / sum over the fragment's rows and the 4 lane quads,
-//   O^T += V^T P^T   with the fp32 weights split into bf16 hi + lo parts (two products): 16 mantissa bits of P
-//                    reach the accumulator, below the bf16 rounding of V and of the stored output.
+//   O += P V         with the fp32 weights split into bf16 hi + lo parts (two products): 16 mantissa bits of P
+//                    reach the accumulator, below the bf16 rounding of V and of the stored output.  O's fragment
+//                    rows are queries 4*(lane/16)+i: their rescale factors come from the lanes that own them.
 template <int NKM, int NVM>
 __global__ void __launch_bounds__(256, 3)
 sink_attn_prefill_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_cache,
@@ -260,9 +264,9 @@ sink_attn_prefill_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict
   const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
   const int ql = lane & 15, quad = lane >> 4;
   const int nk = d >> 4, nv = vd >> 4;
-  const int kstride = d + 8, vstride = KT + 4;
+  const int kstride = d + 8, vstride = vd + 8;
   short* Ks = reinterpret_cast<short*>(smem_raw);  // [KT][d+8] bf16 bits
-  short* Vt = Ks + KT * kstride;                   // [vd][KT+4]
+  short* Vs = Ks + KT * kstride;                   // [KT][vd+8]
   const int tq = q0 + wid * 16 + ql;               // this lane's query (a fragment column)
   const bool q_ok = tq < qlen;
   bf16x4_t qf[NKM];
@@ -305,8 +309,7 @@ sink_attn_prefill_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict
         if (blk >= 0 && blk < nblocks)
           v = *reinterpret_cast<const bf16x8_t*>(v_cache + (((size_t)blk * G + g) * BS + key % BS) * vd + c * 8);
       }
-#pragma unroll
-      for (int e = 0; e < 8; ++e) Vt[(c * 8 + e) * vstride + kk] = v[e];
+      *reinterpret_cast<bf16x8_t*>(Vs + kk * vstride + c * 8) = v;
     }
     __syncthreads();
     if (k0 > wave_qmax) continue;  // every key of the tile lies after this wave's queries
@@ -350,8 +353,13 @@ sink_attn_prefill_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict
     psum += __shfl_xor(psum, 32, 64);
     l = l * alpha + psum;
     m = mn;
+    float arow[4];  // the rescale factors of this lane's accumulator rows (queries 4*quad + i)
 #pragma unroll
-    for (int v = 0; v < NVM; ++v) acc[v] *= alpha;
+    for (int i = 0; i < 4; ++i) arow[i] = __shfl(alpha, 4 * quad + i, 64);
+#pragma unroll
+    for (int v = 0; v < NVM; ++v)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[v][i] *= arow[i];
 #pragma unroll
     for (int n = 0; n < 4; ++n) {
       bf16x4_t ph, pl;
@@ -361,27 +369,29 @@ sink_attn_prefill_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict
         ph[j] = hi;
         pl[j] = f2bits(st[n][j] - bits2f(hi));
       }
+      const short* vr = Vs + (16 * n + 4 * quad) * vstride + ql;
 #pragma unroll
       for (int v = 0; v < NVM; ++v) {
         if (v < nv) {
-          const bf16x4_t a = *reinterpret_cast<const bf16x4_t*>(Vt + (16 * v + ql) * vstride + 16 * n + 4 * quad);
-          acc[v] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, ph, acc[v], 0, 0, 0);
-          acc[v] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, pl, acc[v], 0, 0, 0);
+          bf16x4_t b;  // V[key 16n + 4*quad + j][value dim 16v + ql]
+#pragma unroll
+          for (int j = 0; j < 4; ++j) b[j] = vr[j * vstride + 16 * v];
+          acc[v] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(ph, b, acc[v], 0, 0, 0);
+          acc[v] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(pl, b, acc[v], 0, 0, 0);
         }
       }
     }
   }
-  if (q_ok) {
-    const float r = out_scale / l;
-    bf16* orow = out + (size_t)(qa + tq) * out_ld + h * vd;
 #pragma unroll
-    for (int v = 0; v < NVM; ++v) {
-      if (v < nv) {
-        bf16x4_t o;
+  for (int i = 0; i < 4; ++i) {
+    const float li = __shfl(l, 4 * quad + i, 64);
+    const int tr = q0 + wid * 16 + 4 * quad + i;  // the query of accumulator row i
+    if (tr < qlen) {
+      const float r = out_scale / li;
+      bf16* orow = out + (size_t)(qa + tr) * out_ld + h * vd + ql;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) o[i] = f2bits(acc[v][i] * r);
-        *reinterpret_cast<bf16x4_t*>(orow + 16 * v + 4 * quad) = o;
-      }
+      for (int v = 0; v < NVM; ++v)
+        if (v < nv) orow[16 * v] = (bf16)(acc[v][i] * r);
     }
   }
 }
@@ -793,8 +803,9 @@ decay_attn_scan_kernel(const T* __restrict__ proj, int ld, int qoff, int koff, i
                                        const int* __restrict__ ctx_len, float* __restrict__ out, int H, int d, int vd,
                                        int nslots, float* __restrict__ ws, int maxchunks) {
   constexpr int TB = 16;
-  extern __shared__ __attribute__((aligned(16))) float smem[];  // [TB][2][dp], dp = d rounded up to 4 (16-B rows)
-  const int dp = (d + 3) & ~3;
+  extern __shared__ __attribute__((aligned(16))) float smem[];  // [TB][2][dp] q | k, then [TB][vd] v
+  const int dp = (d + 3) & ~3;  // d rounded up to 4 (16-B rows)
+  float* vsm = smem + TB * 2 * dp;
   const int seq = blockIdx.y, h = blockIdx.x;
   int qa = q_start[seq], qlen = q_start[seq + 1] - qa;
   if (qlen <= 0) return;
@@ -827,11 +838,15 @@ decay_attn_scan_kernel(const T* __restrict__ proj, int ld, int qoff, int koff, i
       const T* row = proj + (size_t)(qa + t0 + tt) * ld + (which ? koff : qoff) + h * d;
       smem[(tt * 2 + which) * dp + i] = silu_acc(ldf(row + i));
     }
+    for (int idx = threadIdx.x; idx < nb * vd; idx += blockDim.x) {
+      const int tt = idx / vd, i = idx - tt * vd;
+      vsm[idx] = silu_acc(ldf(proj + (size_t)(qa + t0 + tt) * ld + voff + h * vd + i));
+    }
     __syncthreads();
     if (j < vd) {
       for (int tt = 0; tt < nb; ++tt) {
         const size_t tok = (size_t)(qa + t0 + tt);
-        const float vj = silu_acc(ldf(proj + tok * ld + voff + h * vd + j));
+        const float vj = vsm[tt * vd + j];
         const f32x4_t* qs = reinterpret_cast<const f32x4_t*>(smem + tt * 2 * dp);
         const f32x4_t* ks = reinterpret_cast<const f32x4_t*>(smem + (tt * 2 + 1) * dp);
         float o = 0.f;
@@ -862,7 +877,7 @@ decay_attn_scan_kernel(const T* __restrict__ proj, int ld, int qoff, int koff, i
 }
 
 // ws[seq, c] (chunk c's own contribution) -> the state at the start of chunk c; the slot's state <- the state after
-// the last chunk.  grid (H, nseq), threads stride over the d * vd elements.
+// the last chunk.  grid (H, nseq, ceil(d * vd / 256)): one thread per state element.
 __global__ void decay_chunk_prefix_kernel(const float* __restrict__ decay, float* __restrict__ state,
                                           const int* __restrict__ slots, const int* __restrict__ q_start,
                                           const int* __restrict__ ctx_len, float* __restrict__ ws, int maxchunks,
@@ -878,16 +893,27 @@ __global__ void decay_chunk_prefix_kernel(const float* __restrict__ decay, float
   const int nch = (qlen + DECAY_CHUNK - 1) / DECAY_CHUNK;
   const float full = powf(lam, (float)DECAY_CHUNK), last = powf(lam, (float)(qlen - (nch - 1) * DECAY_CHUNK));
   const size_t cs = (size_t)H * d * vd;
-  for (int e = threadIdx.x; e < d * vd; e += blockDim.x) {
-    float S = fresh ? 0.f : Sg[e];
-    float* w = ws + ((size_t)seq * maxchunks * H + h) * d * vd + e;
-    for (int c = 0; c < nch; ++c) {
-      const float u = w[c * cs];
-      w[c * cs] = S;
-      S = fmaf(c == nch - 1 ? last : full, S, u);
+  const int e = blockIdx.z * blockDim.x + threadIdx.x;  // grid.z covers the d * vd elements
+  if (e >= d * vd) return;
+  float S = fresh ? 0.f : Sg[e];
+  float* w = ws + ((size_t)seq * maxchunks * H + h) * d * vd + e;
+  int c = 0;
+  for (; c + 4 <= nch - 1; c += 4) {  // four chunks' loads in flight at once (none of them the last chunk)
+    float u[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) u[k] = w[(c + k) * cs];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      w[(c + k) * cs] = S;
+      S = fmaf(full, S, u[k]);
     }
-    Sg[e] = S;
   }
+  for (; c < nch; ++c) {
+    const float u = w[c * cs];
+    w[c * cs] = S;
+    S = fmaf(c == nch - 1 ? last : full, S, u);
+  }
+  Sg[e] = S;
 }
 
 // out [T, out_ld slice] = out_scale * x / rms(x) * w * sigmoid(gate), x fp32 [T, N]; gate at proj column goff.
@@ -942,7 +968,7 @@ __global__ void mingru_scan_kernel(const T* __restrict__ proj, int ld, int zoff,
 //   pass 1 (PASS = 1): every (sequence, chunk, channel) writes its (A, B) to ws [nseq * maxchunks, 2, W];
 //   pass 2 (PASS = 2): every chunk folds the (A, B) of the chunks before it onto the slot's state (<= maxchunks
 //                      steps), then walks its tokens again and writes the outputs; the last chunk stores the state.
-constexpr int MINGRU_CHUNK = 64;
+constexpr int MINGRU_CHUNK = 32;
 
 template <typename T, int PASS>
 __global__ void mingru_chunk_kernel(const T* __restrict__ proj, int ld, int zoff, int xoff, int goff,
@@ -965,6 +991,7 @@ __global__ void mingru_chunk_kernel(const T* __restrict__ proj, int ld, int zoff
     S = (ctx_len[seq] - qlen == 0 || !slot_ok) ? 0.f : state[(size_t)slot * W + c];
     for (int k = 0; k < ch; ++k) S = fmaf(w[(size_t)k * 2 * W + c], S, w[(size_t)k * 2 * W + W + c]);
   }
+#pragma unroll 8
   for (int t = 0; t < n; ++t) {
     const T* row = proj + (size_t)(qa + t0 + t) * ld;
     const float z = sigmoid_acc(ldf(row + zoff + c) + zb);
@@ -987,12 +1014,30 @@ __global__ void mingru_chunk_kernel(const T* __restrict__ proj, int ld, int zoff
 // gu [T, 2F] (gate | up): y = g sigmoid(alpha g) (u + 1), g = min(gate, limit), u = clamp(up, -limit, limit).
 template <typename T>
 __global__ void clamped_glu_kernel(const T* __restrict__ gu, T* __restrict__ out, int F, float limit, float alpha) {
-  const size_t t = blockIdx.y;
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t t = blockIdx.x;
+  const int i = blockIdx.y * blockDim.x + threadIdx.x;
   if (i >= F) return;
   const float g = fminf(ldf(gu + t * 2 * F + i), limit);
   const float u = fminf(fmaxf(ldf(gu + t * 2 * F + F + i), -limit), limit);
   stf(out + t * F + i, g * sigmoid_acc(alpha * g) * (u + 1.f));
+}
+
+// bf16, F % 8 == 0: 16-byte loads and stores, 8 elements per thread
+__global__ void clamped_glu_vec_kernel(const bf16* __restrict__ gu, bf16* __restrict__ out, int F, float limit,
+                                       float alpha) {
+  const size_t t = blockIdx.x;
+  const int i = (blockIdx.y * blockDim.x + threadIdx.x) * 8;
+  if (i >= F) return;
+  const bf16x8_t g8 = *reinterpret_cast<const bf16x8_t*>(gu + t * 2 * F + i);
+  const bf16x8_t u8 = *reinterpret_cast<const bf16x8_t*>(gu + t * 2 * F + F + i);
+  bf16x8_t o;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const float g = fminf(bits2f(g8[e]), limit);
+    const float u = fminf(fmaxf(bits2f(u8[e]), -limit), limit);
+    o[e] = f2bits(g * sigmoid_acc(alpha * g) * (u + 1.f));
+  }
+  *reinterpret_cast<bf16x8_t*>(out + t * F + i) = o;
 }
 
 }  // namespace grag
@@ -1020,7 +1065,7 @@ GRAG_API hipError_t grag_dyt_residual(const void* y, float a1, const float* w1, 
                                       const float* add_rows, const float* add_vec, float a2, const float* w2,
                                       const float* b2, void* out, int T_, int H, int dt, hipStream_t st) {
   if (T_ <= 0) return hipSuccess;
-  DT_DISPATCH(dt, hipLaunchKernelGGL(dyt_residual_kernel<T>, dim3(T_), dim3(256), 0, st, (const T*)y, a1, w1, b1,
+  DT_DISPATCH(dt, hipLaunchKernelGGL(dyt_residual_kernel<T>, dim3(T_, (H + 1023) / 1024), dim3(256), 0, st, (const T*)y, a1, w1, b1,
                                      resid, add_rows, add_vec, a2, w2, b2, (T*)out, H);)
   return hipGetLastError();
 }
@@ -1030,7 +1075,8 @@ GRAG_API hipError_t grag_rope_vnorm_store(const void* proj, int ld, int qoff, in
                                           void* k_cache, void* v_cache, int T_, int H, int G, int d, int vd, int rd,
                                           int BS, long nslots, float eps, int dt, hipStream_t st) {
   if (T_ <= 0) return hipSuccess;
-  DT_DISPATCH(dt, hipLaunchKernelGGL(rope_vnorm_store_kernel<T>, dim3(T_), dim3(256), 0, st, (const T*)proj, ld, qoff,
+  if (H + 2 * G > 65535) return hipErrorInvalidValue;
+  DT_DISPATCH(dt, hipLaunchKernelGGL(rope_vnorm_store_kernel<T>, dim3(T_, H + 2 * G), dim3(64), 0, st, (const T*)proj, ld, qoff,
                                      koff, voff, positions, table, table_rows, slot_mapping, (T*)q_out, (T*)k_cache,
                                      (T*)v_cache, H, G, d, vd, rd, BS, nslots, eps);)
   return hipGetLastError();
@@ -1057,7 +1103,7 @@ GRAG_API hipError_t grag_sink_attn_prefill(const void* q, const void* k_cache, c
   if (vd > 64 * SA_VC || G <= 0 || H % G) return hipErrorInvalidValue;
   if (dt == 0 && max_q_len >= 16 && d % 16 == 0 && vd % 16 == 0 && d <= 256 && vd <= 256 && out_ld % 4 == 0 &&
       (reinterpret_cast<uintptr_t>(out) & 7) == 0 && (reinterpret_cast<uintptr_t>(q) & 7) == 0) {
-    const size_t mb = ((size_t)64 * (d + 8) + (size_t)vd * (64 + 4)) * sizeof(short);
+    const size_t mb = ((size_t)64 * (d + 8) + (size_t)64 * (vd + 8)) * sizeof(short);
     const dim3 mgrid((max_q_len + 63) / 64, H, nseq);
 #define SA_MFMA(NK, NV)                                                                                              \
   {                                                                                                                  \
@@ -1155,7 +1201,7 @@ static hipError_t launch_decay_scan(const T* proj, int ld, int qoff, int koff, i
                                     int nseq, int H, int d, int vd, int nslots, float* ws, int maxchunks,
                                     hipStream_t st) {
   const int threads = ((vd + 63) / 64) * 64;
-  const size_t bytes = (size_t)16 * 2 * ((d + 3) & ~3) * sizeof(float);
+  const size_t bytes = (size_t)16 * (2 * ((d + 3) & ~3) + vd) * sizeof(float);
   const dim3 grid(H, nseq, MODE == 0 ? 1 : maxchunks);
 #define DECAY_LAUNCH(DM)                                                                                     \
   hipLaunchKernelGGL((decay_attn_scan_kernel<T, DM, MODE>), grid, dim3(threads), bytes, st, proj, ld, qoff, koff, \
@@ -1194,7 +1240,7 @@ GRAG_API hipError_t grag_decay_attn_scan(const void* proj, int ld, int qoff, int
   DT_DISPATCH(dt, e = (launch_decay_scan<T, 1>((const T*)proj, ld, qoff, koff, voff, decay, state, slots, q_start,
                                                ctx_len, out, nseq, H, d, vd, nslots, ws, maxchunks, st));)
   if (e != hipSuccess) return e;
-  hipLaunchKernelGGL(decay_chunk_prefix_kernel, dim3(H, nseq), dim3(256), 0, st, decay, state, slots, q_start, ctx_len,
+  hipLaunchKernelGGL(decay_chunk_prefix_kernel, dim3(H, nseq, (d * vd + 255) / 256), dim3(256), 0, st, decay, state, slots, q_start, ctx_len,
                      ws, maxchunks, H, d, vd, nslots);
   DT_DISPATCH(dt, e = (launch_decay_scan<T, 2>((const T*)proj, ld, qoff, koff, voff, decay, state, slots, q_start,
                                                ctx_len, out, nseq, H, d, vd, nslots, ws, maxchunks, st));)
@@ -1238,7 +1284,12 @@ GRAG_API hipError_t grag_mingru_scan(const void* proj, int ld, int zoff, int xof
 GRAG_API hipError_t grag_clamped_glu(const void* gu, void* out, int T_, int F, float limit, float alpha, int dt,
                                      hipStream_t st) {
   if (T_ <= 0) return hipSuccess;
-  const dim3 grid((F + 255) / 256, T_);
+  if (dt == 0 && F % 8 == 0 && (reinterpret_cast<uintptr_t>(gu) & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0) {
+    hipLaunchKernelGGL(clamped_glu_vec_kernel, dim3(T_, (F / 8 + 255) / 256), dim3(256), 0, st, (const bf16*)gu,
+                       (bf16*)out, F, limit, alpha);
+    return hipGetLastError();
+  }
+  const dim3 grid(T_, (F + 255) / 256);
   DT_DISPATCH(dt, hipLaunchKernelGGL(clamped_glu_kernel<T>, grid, dim3(256), 0, st, (const T*)gu, (T*)out, F, limit,
                                      alpha);)
   return hipGetLastError();
