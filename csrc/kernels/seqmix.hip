@@ -239,6 +239,39 @@ sink_attn_prefill_kernel(const T* __restrict__ q, const T* __restrict__ k_cache,
   }
 }
 
+// ---- 64-key tiles of the paged K / V caches for the matrix-core attention kernels: each of the 256 threads carries
+// NL 16-byte vectors of a tile in registers (rows of `rowlen` bf16, rowlen % 8 == 0), loaded one tile AHEAD of the
+// tile being computed, then stored row-major into LDS (row stride `stride`, a multiple of 8).
+template <int NL>
+__device__ __forceinline__ void tile_load(bf16x8_t (&reg)[NL], const bf16* __restrict__ cache,
+                                          const int* __restrict__ bt, int k0, int kend, int rowlen, int G, int g,
+                                          int BS, int nblocks, unsigned code) {
+  const int r8 = rowlen >> 3;
+#pragma unroll
+  for (int u = 0; u < NL; ++u) {
+    reg[u] = bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
+    const int idx = threadIdx.x + u * 256;
+    const int kk = idx / r8, c = idx - kk * r8;
+    const int key = k0 + kk;
+    if (kk < 64 && key < kend) {
+      const int blk = bt[key / BS];
+      if (index_ok(blk, nblocks, code))
+        reg[u] = *reinterpret_cast<const bf16x8_t*>(cache + (((size_t)blk * G + g) * BS + key % BS) * rowlen + c * 8);
+    }
+  }
+}
+template <int NL>
+__device__ __forceinline__ void tile_store(const bf16x8_t (&reg)[NL], short* __restrict__ dst, int rowlen,
+                                           int stride) {
+  const int r8 = rowlen >> 3;
+#pragma unroll
+  for (int u = 0; u < NL; ++u) {
+    const int idx = threadIdx.x + u * 256;
+    const int kk = idx / r8, c = idx - kk * r8;
+    if (kk < 64) *reinterpret_cast<bf16x8_t*>(dst + kk * stride + c * 8) = reg[u];
+  }
+}
+
 // prefill on the matrix cores (bf16 activations, d and vd multiples of 16): grid (tiles of 64 queries, H, nseq), 4 waves
 // of 16 queries.  Per 64-key tile (K [64][d+8] and V [64][vd+8] staged in LDS as bf16, both row-major):
 //   S^T = K Q^T      v_mfma_f32_16x16x16_bf16: bf16 products are exact in fp32, fp32 accumulation; the C fragment
@@ -259,7 +292,9 @@ sink_attn_prefill_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
   const int seq = blockIdx.z, h = blockIdx.y, g = h / (H / G);
   const int qa = q_start[seq], qlen = q_start[seq + 1] - qa, ctx = ctx_len[seq];
-  const int q0 = blockIdx.x * 64;
+  // query tile of this block, rotated by the head: workgroups that land on one CU together (ids a multiple of the CU
+  // count apart) then hold query tiles of different causal lengths instead of four of the longest
+  const int q0 = (int)((blockIdx.x + 9u * blockIdx.y + 5u * blockIdx.z) % gridDim.x) * 64;
   if (q0 >= qlen) return;
   const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
   const int ql = lane & 15, quad = lane >> 4;
@@ -285,33 +320,18 @@ sink_attn_prefill_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict
   const int nkeys = min(ctx, pos0 + min(q0 + 64, qlen));
   const int wave_qmax = pos0 + min(q0 + wid * 16 + 15, qlen - 1);
   const int* bt = block_tables + (size_t)seq * bt_stride;
-  const int dv8 = d >> 3, vv8 = vd >> 3;
+  bf16x8_t kreg[NKM / 2], vreg[NVM / 2];
+  tile_load(kreg, k_cache, bt, 0, nkeys, d, G, g, BS, nblocks, ERR_BLOCK_PREFILL);
+  tile_load(vreg, v_cache, bt, 0, nkeys, vd, G, g, BS, nblocks, ERR_BLOCK_PREFILL);
   for (int k0 = 0; k0 < nkeys; k0 += KT) {
     __syncthreads();
-    const int kn = min(KT, nkeys - k0);
-    for (int idx = threadIdx.x; idx < KT * dv8; idx += 256) {
-      const int kk = idx / dv8, c = idx - kk * dv8;
-      bf16x8_t v = bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
-      if (kk < kn) {
-        const int key = k0 + kk;
-        const int blk = bt[key / BS];
-        if (index_ok(blk, nblocks, ERR_BLOCK_PREFILL))
-          v = *reinterpret_cast<const bf16x8_t*>(k_cache + (((size_t)blk * G + g) * BS + key % BS) * d + c * 8);
-      }
-      *reinterpret_cast<bf16x8_t*>(Ks + kk * kstride + c * 8) = v;
-    }
-    for (int idx = threadIdx.x; idx < KT * vv8; idx += 256) {
-      const int kk = idx / vv8, c = idx - kk * vv8;
-      bf16x8_t v = bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
-      if (kk < kn) {
-        const int key = k0 + kk;
-        const int blk = bt[key / BS];
-        if (blk >= 0 && blk < nblocks)
-          v = *reinterpret_cast<const bf16x8_t*>(v_cache + (((size_t)blk * G + g) * BS + key % BS) * vd + c * 8);
-      }
-      *reinterpret_cast<bf16x8_t*>(Vs + kk * vstride + c * 8) = v;
-    }
+    tile_store(kreg, Ks, d, kstride);
+    tile_store(vreg, Vs, vd, vstride);
     __syncthreads();
+    if (k0 + KT < nkeys) {  // the next tile's loads fly while this one is computed
+      tile_load(kreg, k_cache, bt, k0 + KT, nkeys, d, G, g, BS, nblocks, ERR_BLOCK_PREFILL);
+      tile_load(vreg, v_cache, bt, k0 + KT, nkeys, vd, G, g, BS, nblocks, ERR_BLOCK_PREFILL);
+    }
     if (k0 > wave_qmax) continue;  // every key of the tile lies after this wave's queries
     f32x4_t st[4];
 #pragma unroll
@@ -326,12 +346,14 @@ sink_attn_prefill_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict
       }
     }
     float tmax = -INFINITY;
+    // a tile wholly at or before the wave's first query (and inside the context) needs no mask
+    const bool interior = k0 + KT - 1 <= pos0 + q0 + wid * 16 && k0 + KT <= nkeys && q0 + wid * 16 + 15 < qlen;
 #pragma unroll
     for (int n = 0; n < 4; ++n)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int key = k0 + 16 * n + 4 * quad + i;
-        const bool vis = q_ok && key < nkeys && key <= qpos;
+        const bool vis = interior || (q_ok && key < nkeys && key <= qpos);
         const float sc = vis ? st[n][i] * scale : -INFINITY;
         st[n][i] = sc;
         tmax = fmaxf(tmax, sc);
@@ -339,13 +361,13 @@ sink_attn_prefill_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict
     tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
     const float mn = fmaxf(m, tmax);  // finite: m starts at the sink
-    const float alpha = expf(m - mn);
+    const float alpha = __expf(m - mn);
     float psum = 0.f;
 #pragma unroll
     for (int n = 0; n < 4; ++n)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float p = st[n][i] == -INFINITY ? 0.f : expf(st[n][i] - mn);
+        const float p = __expf(st[n][i] - mn);  // (e^-inf = 0 for masked scores)
         st[n][i] = p;
         psum += p;
       }
@@ -399,7 +421,7 @@ sink_attn_prefill_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict
 // decode on the matrix cores (bf16, d and vd multiples of 16, H / G <= 16): grid (key splits, G, nseq), 4 waves.
 // The 16 fragment columns are the query heads that share one kv head (GQA packing: K / V are read once for all of
 // them).  The block stages 64-key tiles as the prefill kernel does; wave w owns keys 16w .. 16w+15 of every tile with
-// its own running (max, sum, O^T) and the four waves merge through LDS at the end.  With nsplit > 1 every split
+// its own running (max, sum, O) and the four waves merge through LDS at the end.  With nsplit > 1 every split
 // writes its unnormalised O and (max, sum) to part_o [nsplit, nseq, H, vd] / part_ml [nsplit, nseq, H, 2] and
 // sink_attn_combine_kernel merges them; the sink term enters once (split 0, wave 0).
 template <int NKM, int NVM>
@@ -418,9 +440,9 @@ sink_attn_decode_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict_
   const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
   const int ql = lane & 15, quad = lane >> 4;
   const int nk = d >> 4, nv = vd >> 4;
-  const int kstride = d + 8, vstride = KT + 4;
+  const int kstride = d + 8, vstride = vd + 8;
   short* Ks = reinterpret_cast<short*>(smem_raw);
-  short* Vt = Ks + KT * kstride;
+  short* Vs = Ks + KT * kstride;
   const bool col_ok = ql < R;
   const int head = g * R + (col_ok ? ql : 0);
   bf16x4_t qf[NKM];
@@ -438,34 +460,21 @@ sink_attn_decode_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict_
   const int kbeg = nsplit > 1 ? sp * split_len : 0;
   const int kend = nsplit > 1 ? min(ctx, kbeg + split_len) : ctx;
   const int* bt = block_tables + (size_t)seq * bt_stride;
-  const int dv8 = d >> 3, vv8 = vd >> 3;
+  bf16x8_t kreg[NKM / 2], vreg[NVM / 2];
+  if (kbeg < kend) {
+    tile_load(kreg, k_cache, bt, kbeg, kend, d, G, g, BS, nblocks, ERR_BLOCK_DECODE);
+    tile_load(vreg, v_cache, bt, kbeg, kend, vd, G, g, BS, nblocks, ERR_BLOCK_DECODE);
+  }
   for (int k0 = kbeg; k0 < kend; k0 += KT) {
     __syncthreads();
-    const int kn = min(KT, kend - k0);
-    for (int idx = threadIdx.x; idx < KT * dv8; idx += 256) {
-      const int kk = idx / dv8, c = idx - kk * dv8;
-      bf16x8_t v = bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
-      if (kk < kn) {
-        const int key = k0 + kk;
-        const int blk = bt[key / BS];
-        if (index_ok(blk, nblocks, ERR_BLOCK_DECODE))
-          v = *reinterpret_cast<const bf16x8_t*>(k_cache + (((size_t)blk * G + g) * BS + key % BS) * d + c * 8);
-      }
-      *reinterpret_cast<bf16x8_t*>(Ks + kk * kstride + c * 8) = v;
-    }
-    for (int idx = threadIdx.x; idx < KT * vv8; idx += 256) {
-      const int kk = idx / vv8, c = idx - kk * vv8;
-      bf16x8_t v = bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
-      if (kk < kn) {
-        const int key = k0 + kk;
-        const int blk = bt[key / BS];
-        if (blk >= 0 && blk < nblocks)
-          v = *reinterpret_cast<const bf16x8_t*>(v_cache + (((size_t)blk * G + g) * BS + key % BS) * vd + c * 8);
-      }
-#pragma unroll
-      for (int e = 0; e < 8; ++e) Vt[(c * 8 + e) * vstride + kk] = v[e];
-    }
+    tile_store(kreg, Ks, d, kstride);
+    tile_store(vreg, Vs, vd, vstride);
     __syncthreads();
+    if (k0 + KT < kend) {
+      tile_load(kreg, k_cache, bt, k0 + KT, kend, d, G, g, BS, nblocks, ERR_BLOCK_DECODE);
+      tile_load(vreg, v_cache, bt, k0 + KT, kend, vd, G, g, BS, nblocks, ERR_BLOCK_DECODE);
+    }
+    const int kn = min(KT, kend - k0);
     if (16 * wid >= kn) continue;  // this wave's 16 keys lie past the split's end
     f32x4_t st = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -500,21 +509,28 @@ sink_attn_decode_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict_
     psum += __shfl_xor(psum, 32, 64);
     l = l * alpha + psum;
     m = mn;
+    float arow[4];  // rescale factors of the accumulator rows (heads 4*quad + i)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) arow[i] = __shfl(alpha, 4 * quad + i, 64);
+    const short* vr = Vs + (16 * wid + 4 * quad) * vstride + ql;
 #pragma unroll
     for (int v = 0; v < NVM; ++v) {
       if (v < nv) {
-        const bf16x4_t a = *reinterpret_cast<const bf16x4_t*>(Vt + (16 * v + ql) * vstride + 16 * wid + 4 * quad);
-        acc[v] *= alpha;
-        acc[v] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, ph, acc[v], 0, 0, 0);
-        acc[v] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, pl, acc[v], 0, 0, 0);
+        bf16x4_t b;  // V[key 16w + 4*quad + j][value dim 16v + ql]
+#pragma unroll
+        for (int j = 0; j < 4; ++j) b[j] = vr[j * vstride + 16 * v];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[v][i] *= arow[i];
+        acc[v] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(ph, b, acc[v], 0, 0, 0);
+        acc[v] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(pl, b, acc[v], 0, 0, 0);
       }
     }
   }
-  // merge the four waves: (m, l) per column, O^T [vd][16 columns] per wave
+  // merge the four waves: (m, l) per head column, O [16 heads][vd] per wave
   __syncthreads();
   float* Mw = reinterpret_cast<float*>(smem_raw);  // [4][16]
   float* Lw = Mw + 64;                             // [4][16]
-  float* Aw = Lw + 64;                             // [4][vd][16]
+  float* Aw = Lw + 64;                             // [4][16][vd]
   if (quad == 0) {
     Mw[wid * 16 + ql] = m;
     Lw[wid * 16 + ql] = l;
@@ -523,7 +539,7 @@ sink_attn_decode_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict_
   for (int v = 0; v < NVM; ++v)
     if (v < nv)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) Aw[((size_t)wid * vd + 16 * v + 4 * quad + i) * 16 + ql] = acc[v][i];
+      for (int i = 0; i < 4; ++i) Aw[((size_t)wid * 16 + 4 * quad + i) * vd + 16 * v + ql] = acc[v][i];
   __syncthreads();
   float M = -INFINITY;
   for (int w = 0; w < 4; ++w) M = fmaxf(M, Mw[w * 16 + ql]);
@@ -533,32 +549,32 @@ sink_attn_decode_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict_
     f[w] = mw == -INFINITY ? 0.f : expf(mw - M);
     L += Lw[w * 16 + ql] * f[w];
   }
-  if (!col_ok) return;
-#pragma unroll
-  for (int v = 0; v < NVM; ++v) {
-    if (v < nv && (v & 3) == wid) {
-      f32x4_t o;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        float x = 0.f;
-        for (int w = 0; w < 4; ++w) x = fmaf(Aw[((size_t)w * vd + 16 * v + 4 * quad + i) * 16 + ql], f[w], x);
-        o[i] = x;
-      }
-      if (nsplit > 1) {
-        *reinterpret_cast<f32x4_t*>(part_o + (((size_t)sp * nseq + seq) * H + head) * vd + 16 * v + 4 * quad) = o;
-      } else {
-        const float r = out_scale / L;
-        bf16x4_t ob;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) ob[i] = f2bits(o[i] * r);
-        *reinterpret_cast<bf16x4_t*>(out + (size_t)seq * out_ld + head * vd + 16 * v + 4 * quad) = ob;
-      }
-    }
-  }
-  if (nsplit > 1 && wid == 0 && quad == 0) {
+  if (nsplit > 1 && wid == 0 && quad == 0 && col_ok) {
     float* ml = part_ml + (((size_t)sp * nseq + seq) * H + head) * 2;
     ml[0] = M;
     ml[1] = L;
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = 4 * quad + i;  // the head of accumulator row i: its factors live in lane r
+    float fr[4];
+#pragma unroll
+    for (int w = 0; w < 4; ++w) fr[w] = __shfl(f[w], r, 64);
+    const float Lr = __shfl(L, r, 64);
+    if (r >= R) continue;
+    const int hr = g * R + r;
+#pragma unroll
+    for (int v = 0; v < NVM; ++v) {
+      if (v < nv && (v & 3) == wid) {
+        float x = 0.f;
+        for (int w = 0; w < 4; ++w) x = fmaf(Aw[((size_t)w * 16 + r) * vd + 16 * v + ql], fr[w], x);
+        if (nsplit > 1) {
+          part_o[(((size_t)sp * nseq + seq) * H + hr) * vd + 16 * v + ql] = x;
+        } else {
+          out[(size_t)seq * out_ld + hr * vd + 16 * v + ql] = (bf16)(x * (out_scale / Lr));
+        }
+      }
+    }
   }
 }
 
@@ -1154,7 +1170,7 @@ GRAG_API hipError_t grag_sink_attn_decode(const void* q, const void* k_cache, co
   if (dt == 0 && d % 16 == 0 && vd % 16 == 0 && d <= 256 && vd <= 256 && H / G <= 16 && out_ld % 4 == 0 &&
       (reinterpret_cast<uintptr_t>(out) & 7) == 0 && (reinterpret_cast<uintptr_t>(q) & 7) == 0 && nseq <= 65535) {
     if (nsplit < 1 || part_o == nullptr || part_ml == nullptr || split_len % 64) nsplit = 1;
-    const size_t kvb = ((size_t)64 * (d + 8) + (size_t)vd * (64 + 4)) * sizeof(short);
+    const size_t kvb = ((size_t)64 * (d + 8) + (size_t)64 * (vd + 8)) * sizeof(short);
     const size_t mgb = (128 + (size_t)4 * vd * 16) * sizeof(float);
     const size_t mb = kvb > mgb ? kvb : mgb;
     const dim3 mgrid(nsplit, G, nseq);
