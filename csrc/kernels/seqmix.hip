@@ -239,36 +239,57 @@ sink_attn_prefill_kernel(const T* __restrict__ q, const T* __restrict__ k_cache,
   }
 }
 
-// ---- 64-key tiles of the paged K / V caches for the matrix-core attention kernels: each of the 256 threads carries
-// NL 16-byte vectors of a tile in registers (rows of `rowlen` bf16, rowlen % 8 == 0), loaded one tile AHEAD of the
-// tile being computed, then stored row-major into LDS (row stride `stride`, a multiple of 8).
+// ---- 64-key tiles of the paged K / V caches for the matrix-core attention kernels.  Thread t of the 256 owns row
+// t / 4 of a tile (one key) and the 16-byte vectors (t % 4) + 4u of that row, for K and for V alike: one block-table
+// lookup per thread and tile, no integer division in the tile loop (the row's position in the paged cache is kept
+// as (block-table index, offset in block) and stepped by 64 keys).  Tiles are loaded into registers one tile AHEAD
+// of the tile being computed, then stored row-major into LDS (row stride `stride`, a multiple of 8 elements).
+struct RowCursor {
+  int bi, off;  // block-table index and offset within the block of this thread's row
+  int q64, r64;
+  __device__ __forceinline__ void init(int key, int BS) {
+    bi = key / BS;
+    off = key - bi * BS;
+    q64 = 64 / BS;
+    r64 = 64 - q64 * BS;
+  }
+  __device__ __forceinline__ void advance(int BS) {
+    bi += q64;
+    off += r64;
+    if (off >= BS) {
+      off -= BS;
+      ++bi;
+    }
+  }
+};
+// the cache block of the cursor's row (-1: the row lies at or past `kend`, or the table entry is out of range)
+__device__ __forceinline__ int tile_block(const RowCursor& rc, const int* __restrict__ bt, int key, int kend,
+                                          int nblocks, unsigned code) {
+  if (key >= kend) return -1;
+  const int blk = bt[rc.bi];
+  return index_ok(blk, nblocks, code) ? blk : -1;
+}
 template <int NL>
-__device__ __forceinline__ void tile_load(bf16x8_t (&reg)[NL], const bf16* __restrict__ cache,
-                                          const int* __restrict__ bt, int k0, int kend, int rowlen, int G, int g,
-                                          int BS, int nblocks, unsigned code) {
+__device__ __forceinline__ void tile_load(bf16x8_t (&reg)[NL], const bf16* __restrict__ cache, int blk, int off,
+                                          int rowlen, int G, int g, int BS) {
   const int r8 = rowlen >> 3;
+  const bf16* row = cache + (((size_t)(blk < 0 ? 0 : blk) * G + g) * BS + off) * rowlen;
 #pragma unroll
   for (int u = 0; u < NL; ++u) {
+    const int c = (threadIdx.x & 3) + 4 * u;
     reg[u] = bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
-    const int idx = threadIdx.x + u * 256;
-    const int kk = idx / r8, c = idx - kk * r8;
-    const int key = k0 + kk;
-    if (kk < 64 && key < kend) {
-      const int blk = bt[key / BS];
-      if (index_ok(blk, nblocks, code))
-        reg[u] = *reinterpret_cast<const bf16x8_t*>(cache + (((size_t)blk * G + g) * BS + key % BS) * rowlen + c * 8);
-    }
+    if (blk >= 0 && c < r8) reg[u] = *reinterpret_cast<const bf16x8_t*>(row + c * 8);
   }
 }
 template <int NL>
 __device__ __forceinline__ void tile_store(const bf16x8_t (&reg)[NL], short* __restrict__ dst, int rowlen,
                                            int stride) {
   const int r8 = rowlen >> 3;
+  short* row = dst + (threadIdx.x >> 2) * stride;
 #pragma unroll
   for (int u = 0; u < NL; ++u) {
-    const int idx = threadIdx.x + u * 256;
-    const int kk = idx / r8, c = idx - kk * r8;
-    if (kk < 64) *reinterpret_cast<bf16x8_t*>(dst + kk * stride + c * 8) = reg[u];
+    const int c = (threadIdx.x & 3) + 4 * u;
+    if (c < r8) *reinterpret_cast<bf16x8_t*>(row + c * 8) = reg[u];
   }
 }
 
@@ -321,16 +342,23 @@ sink_attn_prefill_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict
   const int wave_qmax = pos0 + min(q0 + wid * 16 + 15, qlen - 1);
   const int* bt = block_tables + (size_t)seq * bt_stride;
   bf16x8_t kreg[NKM / 2], vreg[NVM / 2];
-  tile_load(kreg, k_cache, bt, 0, nkeys, d, G, g, BS, nblocks, ERR_BLOCK_PREFILL);
-  tile_load(vreg, v_cache, bt, 0, nkeys, vd, G, g, BS, nblocks, ERR_BLOCK_PREFILL);
+  RowCursor rc;
+  rc.init(threadIdx.x >> 2, BS);
+  {
+    const int blk = tile_block(rc, bt, threadIdx.x >> 2, nkeys, nblocks, ERR_BLOCK_PREFILL);
+    tile_load(kreg, k_cache, blk, rc.off, d, G, g, BS);
+    tile_load(vreg, v_cache, blk, rc.off, vd, G, g, BS);
+  }
   for (int k0 = 0; k0 < nkeys; k0 += KT) {
     __syncthreads();
     tile_store(kreg, Ks, d, kstride);
     tile_store(vreg, Vs, vd, vstride);
     __syncthreads();
     if (k0 + KT < nkeys) {  // the next tile's loads fly while this one is computed
-      tile_load(kreg, k_cache, bt, k0 + KT, nkeys, d, G, g, BS, nblocks, ERR_BLOCK_PREFILL);
-      tile_load(vreg, v_cache, bt, k0 + KT, nkeys, vd, G, g, BS, nblocks, ERR_BLOCK_PREFILL);
+      rc.advance(BS);
+      const int blk = tile_block(rc, bt, k0 + KT + (threadIdx.x >> 2), nkeys, nblocks, ERR_BLOCK_PREFILL);
+      tile_load(kreg, k_cache, blk, rc.off, d, G, g, BS);
+      tile_load(vreg, v_cache, blk, rc.off, vd, G, g, BS);
     }
     if (k0 > wave_qmax) continue;  // every key of the tile lies after this wave's queries
     f32x4_t st[4];
@@ -461,9 +489,12 @@ sink_attn_decode_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict_
   const int kend = nsplit > 1 ? min(ctx, kbeg + split_len) : ctx;
   const int* bt = block_tables + (size_t)seq * bt_stride;
   bf16x8_t kreg[NKM / 2], vreg[NVM / 2];
+  RowCursor rc;
+  rc.init(kbeg + (threadIdx.x >> 2), BS);
   if (kbeg < kend) {
-    tile_load(kreg, k_cache, bt, kbeg, kend, d, G, g, BS, nblocks, ERR_BLOCK_DECODE);
-    tile_load(vreg, v_cache, bt, kbeg, kend, vd, G, g, BS, nblocks, ERR_BLOCK_DECODE);
+    const int blk = tile_block(rc, bt, kbeg + (threadIdx.x >> 2), kend, nblocks, ERR_BLOCK_DECODE);
+    tile_load(kreg, k_cache, blk, rc.off, d, G, g, BS);
+    tile_load(vreg, v_cache, blk, rc.off, vd, G, g, BS);
   }
   for (int k0 = kbeg; k0 < kend; k0 += KT) {
     __syncthreads();
@@ -471,8 +502,10 @@ sink_attn_decode_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict_
     tile_store(vreg, Vs, vd, vstride);
     __syncthreads();
     if (k0 + KT < kend) {
-      tile_load(kreg, k_cache, bt, k0 + KT, kend, d, G, g, BS, nblocks, ERR_BLOCK_DECODE);
-      tile_load(vreg, v_cache, bt, k0 + KT, kend, vd, G, g, BS, nblocks, ERR_BLOCK_DECODE);
+      rc.advance(BS);
+      const int blk = tile_block(rc, bt, k0 + KT + (threadIdx.x >> 2), kend, nblocks, ERR_BLOCK_DECODE);
+      tile_load(kreg, k_cache, blk, rc.off, d, G, g, BS);
+      tile_load(vreg, v_cache, blk, rc.off, vd, G, g, BS);
     }
     const int kn = min(KT, kend - k0);
     if (16 * wid >= kn) continue;  // this wave's 16 keys lie past the split's end
