@@ -23,6 +23,16 @@ template <> __device__ __forceinline__ void stf<float>(float* p, float v) { *p =
 __device__ __forceinline__ float sigmoidf_(float x) { return 1.f / (1.f + __expf(-x)); }
 __device__ __forceinline__ float sigmoid_acc(float x) { return 1.f / (1.f + expf(-x)); }
 __device__ __forceinline__ float silu_acc(float x) { return x / (1.f + expf(-x)); }
+// tanh in fp32 to a few ulp: (1 - e^-2|x|) / (1 + e^-2|x|), a short odd series below 0.02 where that form cancels
+__device__ __forceinline__ float tanh_acc(float x) {
+  const float a = fabsf(x);
+  if (a < 0.02f) {
+    const float x2 = x * x;
+    return x * (1.f + x2 * (-0.33333334f + x2 * 0.13333334f));
+  }
+  const float t = expf(-2.f * a);
+  return copysignf((1.f - t) / (1.f + t), x);
+}
 
 // ------------------------------------------------------------------------------------------------ embedding
 template <typename T>
@@ -55,11 +65,37 @@ __global__ void dyt_residual_kernel(const T* __restrict__ y, float a1, const flo
     const int i = i0 + k * 256;
     if (i >= H) break;
     float x = resid[base + i];
-    if (y != nullptr) x += tanhf(a1 * ldf(y + base + i)) * w1[i] + b1[i];
+    if (y != nullptr) x += tanh_acc(a1 * ldf(y + base + i)) * w1[i] + b1[i];
     if (add_rows != nullptr) x += add_rows[base + i];
     if (add_vec != nullptr) x += add_vec[i];
     if (y != nullptr || add_rows != nullptr || add_vec != nullptr) resid[base + i] = x;
-    if (out != nullptr) stf(out + base + i, tanhf(a2 * x) * w2[i] + b2[i]);
+    if (out != nullptr) stf(out + base + i, tanh_acc(a2 * x) * w2[i] + b2[i]);
+  }
+}
+
+// H % 4 == 0: four consecutive elements per thread (16-byte loads of the stream and of the norm vectors)
+template <typename T>
+__global__ void dyt_residual_vec_kernel(const T* __restrict__ y, float a1, const float* __restrict__ w1,
+                                        const float* __restrict__ b1, float* __restrict__ resid,
+                                        const float* __restrict__ add_rows, const float* __restrict__ add_vec,
+                                        float a2, const float* __restrict__ w2, const float* __restrict__ b2,
+                                        T* __restrict__ out, int H) {
+  const size_t base = (size_t)blockIdx.x * H;
+  const int i = blockIdx.y * 1024 + threadIdx.x * 4;
+  if (i >= H) return;
+  f32x4_t x = *reinterpret_cast<const f32x4_t*>(resid + base + i);
+  if (y != nullptr) {
+    const f32x4_t w = *reinterpret_cast<const f32x4_t*>(w1 + i), b = *reinterpret_cast<const f32x4_t*>(b1 + i);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) x[e] += tanh_acc(a1 * ldf(y + base + i + e)) * w[e] + b[e];
+  }
+  if (add_rows != nullptr) x += *reinterpret_cast<const f32x4_t*>(add_rows + base + i);
+  if (add_vec != nullptr) x += *reinterpret_cast<const f32x4_t*>(add_vec + i);
+  if (y != nullptr || add_rows != nullptr || add_vec != nullptr) *reinterpret_cast<f32x4_t*>(resid + base + i) = x;
+  if (out != nullptr) {
+    const f32x4_t w = *reinterpret_cast<const f32x4_t*>(w2 + i), b = *reinterpret_cast<const f32x4_t*>(b2 + i);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) stf(out + base + i + e, tanh_acc(a2 * x[e]) * w[e] + b[e]);
   }
 }
 
@@ -67,14 +103,15 @@ __global__ void dyt_residual_kernel(const T* __restrict__ y, float a1, const flo
 // proj [T, ld]: q heads at column qoff (H x d), k heads at koff (G x d), v heads at voff (G x vd).
 // q_out [T, H*d] = rotated q; k_cache [nblk, G, BS, d] <- rotated k; v_cache [nblk, G, BS, vd] <- v / rms(v).
 // Rotation: the first rd dims of a head, dim i paired with i + rd/2; table row p = cos[0:rd/2] | sin[0:rd/2] (fp32).
-// grid (T, H + G + G): one wave per (token, head): q heads, then k heads, then v heads.
+// grid (T, ceil((H + G + G) / 4)), 256 threads: one wave per (token, head): q heads, then k heads, then v heads.
 template <typename T>
 __global__ void rope_vnorm_store_kernel(const T* __restrict__ proj, int ld, int qoff, int koff, int voff,
                                         const int* __restrict__ positions, const float* __restrict__ table,
                                         int table_rows, const int* __restrict__ slot_mapping, T* __restrict__ q_out,
                                         T* __restrict__ k_cache, T* __restrict__ v_cache, int H, int G, int d, int vd,
                                         int rd, int BS, long nslots, float eps) {
-  const int t = blockIdx.x, hb = blockIdx.y, lane = threadIdx.x;
+  const int t = blockIdx.x, hb = blockIdx.y * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (hb >= H + 2 * G) return;
   const T* row = proj + (size_t)t * ld;
   const int slot = slot_mapping[t];
   const bool store = slot >= 0 && index_ok(slot, nslots, ERR_KV_SLOT);
@@ -1114,6 +1151,12 @@ GRAG_API hipError_t grag_dyt_residual(const void* y, float a1, const float* w1, 
                                       const float* add_rows, const float* add_vec, float a2, const float* w2,
                                       const float* b2, void* out, int T_, int H, int dt, hipStream_t st) {
   if (T_ <= 0) return hipSuccess;
+  auto al16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+  if (H % 4 == 0 && al16(resid) && al16(w1) && al16(b1) && al16(w2) && al16(b2) && al16(add_rows) && al16(add_vec)) {
+    DT_DISPATCH(dt, hipLaunchKernelGGL(dyt_residual_vec_kernel<T>, dim3(T_, (H + 1023) / 1024), dim3(256), 0, st,
+                                       (const T*)y, a1, w1, b1, resid, add_rows, add_vec, a2, w2, b2, (T*)out, H);)
+    return hipGetLastError();
+  }
   DT_DISPATCH(dt, hipLaunchKernelGGL(dyt_residual_kernel<T>, dim3(T_, (H + 1023) / 1024), dim3(256), 0, st, (const T*)y, a1, w1, b1,
                                      resid, add_rows, add_vec, a2, w2, b2, (T*)out, H);)
   return hipGetLastError();
@@ -1124,8 +1167,8 @@ GRAG_API hipError_t grag_rope_vnorm_store(const void* proj, int ld, int qoff, in
                                           void* k_cache, void* v_cache, int T_, int H, int G, int d, int vd, int rd,
                                           int BS, long nslots, float eps, int dt, hipStream_t st) {
   if (T_ <= 0) return hipSuccess;
-  if (H + 2 * G > 65535) return hipErrorInvalidValue;
-  DT_DISPATCH(dt, hipLaunchKernelGGL(rope_vnorm_store_kernel<T>, dim3(T_, H + 2 * G), dim3(64), 0, st, (const T*)proj, ld, qoff,
+  if (H + 2 * G > 4 * 65535) return hipErrorInvalidValue;
+  DT_DISPATCH(dt, hipLaunchKernelGGL(rope_vnorm_store_kernel<T>, dim3(T_, (H + 2 * G + 3) / 4), dim3(256), 0, st, (const T*)proj, ld, qoff,
                                      koff, voff, positions, table, table_rows, slot_mapping, (T*)q_out, (T*)k_cache,
                                      (T*)v_cache, H, G, d, vd, rd, BS, nslots, eps);)
   return hipGetLastError();
