@@ -179,8 +179,9 @@ def hybrid_config_from_dict(d: dict, name: str = "zofesun") -> HybridConfig:
         kind, m = e["type"], e["mixer"]
         if kind == "parallel":
             l, r = m["left"], m["right"]
-            left = SinkAttnSpec(int(l["heads"]), int(l["kv_heads"]), int(l["dim"]), int(l["vdim"]), float(l["scale"]),
-                                int(l["rot"]["dims"]), float(l["rot"]["base"]))
+            rot = l.get("rot") or {"dims": 0, "base": 1.0}  # no "rot" entry: no rotation
+            left = SinkAttnSpec(int(l["heads"]), int(l.get("kv_heads", l["heads"])), int(l["dim"]), int(l["vdim"]),
+                                float(l["scale"]), int(rot["dims"]), float(rot.get("base", 1.0)))
             right = DecayAttnSpec(int(r["heads"]), int(r["dim"]), int(r["vdim"]), tuple(float(x) for x in r["decay"]))
             if left.heads % left.kv_heads or left.rot_dims % 2 or left.rot_dims > left.dim:
                 raise ValueError(f"bad attention sizes {l}")
