@@ -330,9 +330,26 @@ __device__ __forceinline__ void tile_store(const bf16x8_t (&reg)[NL], short* __r
   }
 }
 
+// V tiles are stored for the B fragment of P V: [16 groups of 4 keys][vd][4 keys] (group stride vd * 4 + 8), so a lane's
+// four keys at one value dim are 8 contiguous bytes.
+template <int NL>
+__device__ __forceinline__ void tile_store_v4(const bf16x8_t (&reg)[NL], short* __restrict__ dst, int vd, int gstride) {
+  const int r8 = vd >> 3;
+  const int kk = threadIdx.x >> 2;
+  short* grp = dst + (kk >> 2) * gstride + (kk & 3);
+#pragma unroll
+  for (int u = 0; u < NL; ++u) {
+    const int c = (threadIdx.x & 3) + 4 * u;
+    if (c < r8) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) grp[(c * 8 + e) * 4] = reg[u][e];
+    }
+  }
+}
+
 // prefill on the matrix cores (bf16 activations, d and vd multiples of 16): grid (tiles of 64 queries, H, nseq), 4 waves
-// of 16 queries.  Per 64-key tile (K [64][d+8] and V [64][vd+8] staged in LDS as bf16, both row-major):
-//   S^T = K Q^T      v_mfma_f32_16x16x16_bf16: bf16 products are exact in fp32, fp32 accumulation; the C fragment
+// of 16 queries.  Per 64-key tile (K [64][d+8] row-major and V in 4-key groups, staged in LDS as bf16):
+//   S^T = K Q^T      v_mfma_f32_16x16x32_bf16: bf16 products are exact in fp32, fp32 accumulation; the C fragment
 //                    (rows = keys 4*(lane/16)+i, column = query lane%16) is, read as "row = query lane%16, k = keys
 //                    4*(lane/16)+i", exactly the A fragment of the next product: P never leaves the registers,
 //   softmax in fp32  per query = per lane column: max / sum over the fragment's rows and the 4 lane quads,
@@ -340,7 +357,7 @@ __device__ __forceinline__ void tile_store(const bf16x8_t (&reg)[NL], short* __r
 //                    reach the accumulator, below the bf16 rounding of V and of the stored output.  O's fragment
 //                    rows are queries 4*(lane/16)+i: their rescale factors come from the lanes that own them.
 template <int NKM, int NVM>
-__global__ void __launch_bounds__(256, 3)
+__global__ void __launch_bounds__(256, NKM <= 8 && NVM <= 8 ? 3 : 2)
 sink_attn_prefill_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_cache,
                               const bf16* __restrict__ v_cache, bf16* __restrict__ out, int out_ld,
                               const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ q_start,
@@ -357,21 +374,28 @@ sink_attn_prefill_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict
   const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
   const int ql = lane & 15, quad = lane >> 4;
   const int nk = d >> 4, nv = vd >> 4;
-  const int kstride = d + 8, vstride = vd + 8;
+  const int kstride = d + 8, vstride = vd * 4 + 8;  // vstride: one 4-key group of V
   short* Ks = reinterpret_cast<short*>(smem_raw);  // [KT][d+8] bf16 bits
-  short* Vs = Ks + KT * kstride;                   // [KT][vd+8]
+  short* Vs = Ks + KT * kstride;                   // [16][vd][4] (+8 per group)
   const int tq = q0 + wid * 16 + ql;               // this lane's query (a fragment column)
   const bool q_ok = tq < qlen;
-  bf16x4_t qf[NKM];
+  // q fragments of the 32-wide dim steps (lane: dims 32s + 8*quad .. +7) and of a 16-wide tail when d / 16 is odd
+  const int nk2 = nk >> 1;
+  bf16x8_t qf[NKM / 2];
+  bf16x4_t qt = bf16x4_t{0, 0, 0, 0};
+  const bf16* qrow = q + ((size_t)(qa + (q_ok ? tq : 0)) * H + h) * d;
 #pragma unroll
-  for (int ks = 0; ks < NKM; ++ks) {
-    qf[ks] = bf16x4_t{0, 0, 0, 0};
-    if (ks < nk && q_ok)
-      qf[ks] = *reinterpret_cast<const bf16x4_t*>(q + ((size_t)(qa + tq) * H + h) * d + ks * 16 + quad * 4);
+  for (int ks = 0; ks < NKM / 2; ++ks) {
+    qf[ks] = bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
+    if (ks < nk2 && q_ok) qf[ks] = *reinterpret_cast<const bf16x8_t*>(qrow + ks * 32 + quad * 8);
   }
+  if ((nk & 1) && q_ok) qt = *reinterpret_cast<const bf16x4_t*>(qrow + (nk - 1) * 16 + quad * 4);
   const int pos0 = ctx - qlen;
   const int qpos = pos0 + tq;
-  float m = sinks[h], l = 1.f;
+  // scores are kept in the log2 domain (one multiply by scale * log2 e, then v_exp_f32): m is the running max there
+  const float LOG2E = 1.4426950408889634f;
+  const float sc2 = scale * LOG2E;
+  float m = sinks[h] * LOG2E, l = 1.f;
   f32x4_t acc[NVM];
 #pragma unroll
   for (int v = 0; v < NVM; ++v) acc[v] = f32x4_t{0.f, 0.f, 0.f, 0.f};
@@ -389,7 +413,7 @@ sink_attn_prefill_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict
   for (int k0 = 0; k0 < nkeys; k0 += KT) {
     __syncthreads();
     tile_store(kreg, Ks, d, kstride);
-    tile_store(vreg, Vs, vd, vstride);
+    tile_store_v4(vreg, Vs, vd, vstride);
     __syncthreads();
     if (k0 + KT < nkeys) {  // the next tile's loads fly while this one is computed
       rc.advance(BS);
@@ -402,37 +426,52 @@ sink_attn_prefill_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict
 #pragma unroll
     for (int n = 0; n < 4; ++n) {
       st[n] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      const short* kr = Ks + (16 * n + ql) * kstride;
 #pragma unroll
-      for (int ks = 0; ks < NKM; ++ks) {
-        if (ks < nk) {
-          const bf16x4_t a = *reinterpret_cast<const bf16x4_t*>(Ks + (16 * n + ql) * kstride + ks * 16 + quad * 4);
-          st[n] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, qf[ks], st[n], 0, 0, 0);
+      for (int ks = 0; ks < NKM / 2; ++ks) {
+        if (ks < nk2) {
+          const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(kr + ks * 32 + quad * 8);
+          st[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qf[ks], st[n], 0, 0, 0);
         }
+      }
+      if (nk & 1) {
+        const bf16x4_t a = *reinterpret_cast<const bf16x4_t*>(kr + (nk - 1) * 16 + quad * 4);
+        st[n] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, qt, st[n], 0, 0, 0);
       }
     }
     float tmax = -INFINITY;
     // a tile wholly at or before the wave's first query (and inside the context) needs no mask
     const bool interior = k0 + KT - 1 <= pos0 + q0 + wid * 16 && k0 + KT <= nkeys && q0 + wid * 16 + 15 < qlen;
+    if (interior) {
 #pragma unroll
-    for (int n = 0; n < 4; ++n)
+      for (int n = 0; n < 4; ++n)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int key = k0 + 16 * n + 4 * quad + i;
-        const bool vis = interior || (q_ok && key < nkeys && key <= qpos);
-        const float sc = vis ? st[n][i] * scale : -INFINITY;
-        st[n][i] = sc;
-        tmax = fmaxf(tmax, sc);
-      }
+        for (int i = 0; i < 4; ++i) {
+          st[n][i] *= sc2;
+          tmax = fmaxf(tmax, st[n][i]);
+        }
+    } else {
+#pragma unroll
+      for (int n = 0; n < 4; ++n)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int key = k0 + 16 * n + 4 * quad + i;
+          const bool vis = q_ok && key < nkeys && key <= qpos;
+          st[n][i] = vis ? st[n][i] * sc2 : -INFINITY;
+          tmax = fmaxf(tmax, st[n][i]);
+        }
+    }
     tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
     const float mn = fmaxf(m, tmax);  // finite: m starts at the sink
-    const float alpha = __expf(m - mn);
+    const bool moved = mn > m;
+    const float alpha = __builtin_amdgcn_exp2f(m - mn);
     float psum = 0.f;
 #pragma unroll
     for (int n = 0; n < 4; ++n)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float p = __expf(st[n][i] - mn);  // (e^-inf = 0 for masked scores)
+        const float p = __builtin_amdgcn_exp2f(st[n][i] - mn);  // (2^-inf = 0 for masked scores)
         st[n][i] = p;
         psum += p;
       }
@@ -440,31 +479,35 @@ sink_attn_prefill_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict
     psum += __shfl_xor(psum, 32, 64);
     l = l * alpha + psum;
     m = mn;
-    float arow[4];  // the rescale factors of this lane's accumulator rows (queries 4*quad + i)
+    if (__any(moved)) {  // some query's max moved: rescale the accumulator rows (queries 4*quad + i)
+      float arow[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) arow[i] = __shfl(alpha, 4 * quad + i, 64);
+      for (int i = 0; i < 4; ++i) arow[i] = __shfl(alpha, 4 * quad + i, 64);
 #pragma unroll
-    for (int v = 0; v < NVM; ++v)
+      for (int v = 0; v < NVM; ++v)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) acc[v][i] *= arow[i];
+        for (int i = 0; i < 4; ++i) acc[v][i] *= arow[i];
+    }
 #pragma unroll
-    for (int n = 0; n < 4; ++n) {
-      bf16x4_t ph, pl;
+    for (int np = 0; np < 2; ++np) {  // 32 keys per product: k-slots j < 4 are keys 32np + 4*quad + j, j >= 4 keys + 16
+      bf16x8_t ph, pl;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const short hi = f2bits(st[n][j]);
+      for (int j = 0; j < 8; ++j) {
+        const float p = st[2 * np + (j >> 2)][j & 3];
+        const short hi = f2bits(p);
         ph[j] = hi;
-        pl[j] = f2bits(st[n][j] - bits2f(hi));
+        pl[j] = f2bits(p - bits2f(hi));
       }
-      const short* vr = Vs + (16 * n + 4 * quad) * vstride + ql;
+      const short* vr = Vs + (8 * np + quad) * vstride + ql * 4;
 #pragma unroll
       for (int v = 0; v < NVM; ++v) {
         if (v < nv) {
-          bf16x4_t b;  // V[key 16n + 4*quad + j][value dim 16v + ql]
-#pragma unroll
-          for (int j = 0; j < 4; ++j) b[j] = vr[j * vstride + 16 * v];
-          acc[v] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(ph, b, acc[v], 0, 0, 0);
-          acc[v] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(pl, b, acc[v], 0, 0, 0);
+          // V[keys 32np + 4*quad + 0..3 | + 16][value dim 16v + ql]
+          const bf16x4_t b0 = *reinterpret_cast<const bf16x4_t*>(vr + 64 * v);
+          const bf16x4_t b1 = *reinterpret_cast<const bf16x4_t*>(vr + 4 * vstride + 64 * v);
+          const bf16x8_t b = bf16x8_t{b0[0], b0[1], b0[2], b0[3], b1[0], b1[1], b1[2], b1[3]};
+          acc[v] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ph, b, acc[v], 0, 0, 0);
+          acc[v] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pl, b, acc[v], 0, 0, 0);
         }
       }
     }
@@ -490,7 +533,7 @@ sink_attn_prefill_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict
 // writes its unnormalised O and (max, sum) to part_o [nsplit, nseq, H, vd] / part_ml [nsplit, nseq, H, 2] and
 // sink_attn_combine_kernel merges them; the sink term enters once (split 0, wave 0).
 template <int NKM, int NVM>
-__global__ void __launch_bounds__(256, 3)
+__global__ void __launch_bounds__(256, NKM <= 8 && NVM <= 8 ? 3 : 2)
 sink_attn_decode_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_cache,
                              const bf16* __restrict__ v_cache, bf16* __restrict__ out, int out_ld,
                              const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ ctx_len,
@@ -505,7 +548,7 @@ sink_attn_decode_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict_
   const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
   const int ql = lane & 15, quad = lane >> 4;
   const int nk = d >> 4, nv = vd >> 4;
-  const int kstride = d + 8, vstride = vd + 8;
+  const int kstride = d + 8, vstride = vd * 4 + 8;  // vstride: one 4-key group of V
   short* Ks = reinterpret_cast<short*>(smem_raw);
   short* Vs = Ks + KT * kstride;
   const bool col_ok = ql < R;
@@ -536,7 +579,7 @@ sink_attn_decode_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict_
   for (int k0 = kbeg; k0 < kend; k0 += KT) {
     __syncthreads();
     tile_store(kreg, Ks, d, kstride);
-    tile_store(vreg, Vs, vd, vstride);
+    tile_store_v4(vreg, Vs, vd, vstride);
     __syncthreads();
     if (k0 + KT < kend) {
       rc.advance(BS);
@@ -582,13 +625,12 @@ sink_attn_decode_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict_
     float arow[4];  // rescale factors of the accumulator rows (heads 4*quad + i)
 #pragma unroll
     for (int i = 0; i < 4; ++i) arow[i] = __shfl(alpha, 4 * quad + i, 64);
-    const short* vr = Vs + (16 * wid + 4 * quad) * vstride + ql;
+    const short* vr = Vs + (4 * wid + quad) * vstride + ql * 4;
 #pragma unroll
     for (int v = 0; v < NVM; ++v) {
       if (v < nv) {
-        bf16x4_t b;  // V[key 16w + 4*quad + j][value dim 16v + ql]
-#pragma unroll
-        for (int j = 0; j < 4; ++j) b[j] = vr[j * vstride + 16 * v];
+        // V[keys 16w + 4*quad + 0..3][value dim 16v + ql]
+        const bf16x4_t b = *reinterpret_cast<const bf16x4_t*>(vr + 64 * v);
 #pragma unroll
         for (int i = 0; i < 4; ++i) acc[v][i] *= arow[i];
         acc[v] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(ph, b, acc[v], 0, 0, 0);
@@ -1195,7 +1237,7 @@ GRAG_API hipError_t grag_sink_attn_prefill(const void* q, const void* k_cache, c
   if (vd > 64 * SA_VC || G <= 0 || H % G) return hipErrorInvalidValue;
   if (dt == 0 && max_q_len >= 16 && d % 16 == 0 && vd % 16 == 0 && d <= 256 && vd <= 256 && out_ld % 4 == 0 &&
       (reinterpret_cast<uintptr_t>(out) & 7) == 0 && (reinterpret_cast<uintptr_t>(q) & 7) == 0) {
-    const size_t mb = ((size_t)64 * (d + 8) + (size_t)64 * (vd + 8)) * sizeof(short);
+    const size_t mb = ((size_t)64 * (d + 8) + (size_t)16 * (vd * 4 + 8)) * sizeof(short);
     const dim3 mgrid((max_q_len + 63) / 64, H, nseq);
 #define SA_MFMA(NK, NV)                                                                                              \
   {                                                                                                                  \
@@ -1246,7 +1288,7 @@ GRAG_API hipError_t grag_sink_attn_decode(const void* q, const void* k_cache, co
   if (dt == 0 && d % 16 == 0 && vd % 16 == 0 && d <= 256 && vd <= 256 && H / G <= 16 && out_ld % 4 == 0 &&
       (reinterpret_cast<uintptr_t>(out) & 7) == 0 && (reinterpret_cast<uintptr_t>(q) & 7) == 0 && nseq <= 65535) {
     if (nsplit < 1 || part_o == nullptr || part_ml == nullptr || split_len % 64) nsplit = 1;
-    const size_t kvb = ((size_t)64 * (d + 8) + (size_t)64 * (vd + 8)) * sizeof(short);
+    const size_t kvb = ((size_t)64 * (d + 8) + (size_t)16 * (vd * 4 + 8)) * sizeof(short);
     const size_t mgb = (128 + (size_t)4 * vd * 16) * sizeof(float);
     const size_t mb = kvb > mgb ? kvb : mgb;
     const dim3 mgrid(nsplit, G, nseq);

@@ -49,6 +49,24 @@ def test_greedy_generation(mixed, max_batched):
     C.case_generate("cpu", mixed=mixed, max_batched=max_batched)
 
 
+def test_generation_survives_preemption():
+    """A KV pool too small for all running requests: the scheduler preempts one (pages and slot freed) and
+    recomputes it later from its first token -- its recurrent state restarts from zero with it."""
+    from githubrepostorag_amd.engine.sequence import SamplingParams
+
+    cfg = O.make_config()
+    sd = O.make_weights(cfg, seed=41)
+    _, eng = C.build(cfg, sd, "cpu", slots=3, pool_tokens=96)
+    prompts = [C.tokens(cfg, 5, 90 + i) for i in range(3)]  # admitted together (a page each), then they grow
+    outs = eng.generate(prompts, SamplingParams(max_tokens=40, temperature=0.0, ignore_eos=True))
+    assert eng.sched.num_preemptions > 0
+    for p, c in zip(prompts, outs):
+        logits, _ = O.forward(cfg, sd, p + c.token_ids[:-1])
+        for j, t in enumerate(c.token_ids):
+            row = logits[len(p) - 1 + j]
+            assert float(row.max() - row[t]) < 2e-3 * float(row.std())
+
+
 def test_bf16_close_to_oracle():
     cfg = O.make_config()
     sd = O.make_weights(cfg, seed=23)

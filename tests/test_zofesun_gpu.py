@@ -32,7 +32,7 @@ def test_sink_attention_far_keys_and_page_borders(dtype, tol):
     T.sink_attention_case("cuda", dtype, tol, T=67, far=(0, 3, 4, 63, 64), bs=4)
 
 
-@pytest.mark.parametrize("d,vd", [(32, 48), (64, 16), (128, 128), (16, 256)])
+@pytest.mark.parametrize("d,vd", [(32, 48), (64, 16), (128, 128), (16, 256), (48, 32), (80, 112)])
 def test_sink_attention_matrix_core_shapes(d, vd):
     """bf16 with head sizes in multiples of 16: prompt portions of >= 16 queries run on the matrix cores."""
     T.sink_attention_case("cuda", torch.bfloat16, 0.03, T=150, far=(0, 15, 16, 64, 131), d=d, vd=vd)
