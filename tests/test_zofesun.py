@@ -200,11 +200,11 @@ def recurrent_case(device, dtype, tol):
     from githubrepostorag_amd.ops.attention import AttnMetadata
     from githubrepostorag_amd.ops.recurrent import decay_attention, mingru_scan
 
-    T, H, d, vd, W = 90, 3, 6, 10, 37
+    T, H, d, vd, W = 90, 4, 6, 10, 37
     g = torch.Generator().manual_seed(2)
     proj = torch.randn(T, H * (2 * d + vd) + 5, generator=g)
     proj[3, 2 * H * d + 5:] += 8.0  # a far token with a large value
-    decay = torch.tensor([1.0, 0.05, 0.98])
+    decay = torch.tensor([1.0, 0.05, 0.98, 1e-9])
     x = proj.to(dtype).double()
     q, k, v = (O.silu(x[:, 5:5 + H * d]).view(T, H, d), O.silu(x[:, 5 + H * d:5 + 2 * H * d]).view(T, H, d),
                O.silu(x[:, 5 + 2 * H * d:]).view(T, H, vd))
@@ -229,8 +229,8 @@ def recurrent_case(device, dtype, tol):
             a += n
         err = (torch.cat(outs).double().cpu() - want).abs().max() / want.abs().max()
         assert float(err) < tol, (cuts, float(err))
-        errg = (torch.cat(outg).double().cpu() - wg).abs().max()
-        assert float(errg) < (tol if dtype == torch.float32 else 0.05), (cuts, float(errg))
+        errg = (torch.cat(outg).double().cpu() - wg).abs().max() / wg.abs().max()
+        assert float(errg) < (tol if dtype == torch.float32 else 0.01), (cuts, float(errg))  # (bf16 outputs)
         assert float(S[0].min()) == 9.0 and float(Sg[1].max()) == 9.0  # other slots untouched
 
 
