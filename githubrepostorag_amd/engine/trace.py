@@ -46,7 +46,7 @@ def run_trace(model_dir: str, dtype: str, out_dir: str, max_tokens: int, device:
         if not line:
             continue
         st = json.loads(line)
-        entries = [(e["id"], e["tokens"], e.get("want") or []) for e in st.get("entries", [])]
+        entries = [(e["id"], e["tokens"], e.get("want") or []) for e in st.get("entries", []) if e.get("tokens")]
         logits = eng.feed(entries, st.get("end") or [])
         if logits is not None:
             tmp = os.path.join(out_dir, f".{st['step']}.f32.tmp")
