@@ -1,0 +1,494 @@
+// Glue and attention kernels for decoders with several residual streams and gated, non-softmax attention (gfx950):
+//   * hyper-connection boundary: S fp32 residual streams mixed by an S x S matrix, the sublayer's output added
+//     with one coefficient per stream, the next sublayer's input read out as a weighted sum and RMS-normed,
+//   * query / key RMS norm + paged store for attention whose values are the un-normed keys,
+//   * latent store: RMS-normed latent | rotated shared key part into a one-head paged cache, rotary on the rotated
+//     tail of every (absorbed) query head,
+//   * sliding-window attention with sigmoid weights (no softmax, no normaliser), prefill and decode.
+// Activations are bf16 or fp32 (dt: 0 = bf16, 1 = fp32; the caches hold the same type); streams, norms, scores and
+// attention weights are fp32 in both.
+#include "common.h"
+
+GRAG_ERR_UNIT(gatedmix)
+
+namespace grag {
+
+template <typename T> __device__ __forceinline__ float ldg(const T* p);
+template <> __device__ __forceinline__ float ldg<bf16>(const bf16* p) { return (float)*p; }
+template <> __device__ __forceinline__ float ldg<float>(const float* p) { return *p; }
+template <typename T> __device__ __forceinline__ void stg(T* p, float v);
+template <> __device__ __forceinline__ void stg<bf16>(bf16* p, float v) { *p = (bf16)v; }
+template <> __device__ __forceinline__ void stg<float>(float* p, float v) { *p = v; }
+
+__device__ __forceinline__ float sigmoid_f(float x) { return 1.f / (1.f + expf(-x)); }
+
+// ------------------------------------------------------------------------------------------------ hyper-connections
+// streams [S][T][H] fp32 (in place).  With y: x_t <- sum_s mix[s][t] x_s + outc[t] y, all streams from the old ones.
+// Then u = sum_s inc[s] x_s (inc null: none of the outputs below), out_sum [T][H] <- u (fp32, optional) and
+// out [T][H] <- u / sqrt(mean(u^2) + eps) * w (optional; w holds the norm's full multiplier).
+// grid (T), 256 threads, H floats of LDS.
+constexpr int HC_MAX = 8;
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+hyper_mix_kernel(float* __restrict__ streams, size_t sstride, int S, const T* __restrict__ y,
+                 const float* __restrict__ mix, const float* __restrict__ outc, const float* __restrict__ inc,
+                 const float* __restrict__ w, float eps, T* __restrict__ out, float* __restrict__ out_sum, int H) {
+  extern __shared__ float us[];
+  __shared__ float red[16];
+  const size_t row = (size_t)blockIdx.x * H;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < H; i += 256) {
+    float x[HC_MAX];
+#pragma unroll
+    for (int s = 0; s < HC_MAX; ++s) x[s] = s < S ? streams[s * sstride + row + i] : 0.f;
+    if (y != nullptr) {
+      const float yi = ldg(y + row + i);
+      float n[HC_MAX];
+#pragma unroll
+      for (int t = 0; t < HC_MAX; ++t) {
+        float a = 0.f;
+        if (t < S) {
+#pragma unroll
+          for (int s = 0; s < HC_MAX; ++s)
+            if (s < S) a = fmaf(mix[s * S + t], x[s], a);
+          a = fmaf(outc[t], yi, a);
+          streams[t * sstride + row + i] = a;
+        }
+        n[t] = a;
+      }
+#pragma unroll
+      for (int t = 0; t < HC_MAX; ++t) x[t] = n[t];
+    }
+    if (inc != nullptr) {
+      float u = 0.f;
+#pragma unroll
+      for (int s = 0; s < HC_MAX; ++s)
+        if (s < S) u = fmaf(inc[s], x[s], u);
+      us[i] = u;
+      ss = fmaf(u, u, ss);
+      if (out_sum != nullptr) out_sum[row + i] = u;
+    }
+  }
+  if (inc == nullptr || out == nullptr) return;
+  ss = block_sum(ss, red);
+  const float r = 1.f / sqrtf(ss / (float)H + eps);
+  for (int i = threadIdx.x; i < H; i += 256) stg(out + row + i, us[i] * r * w[i]);
+}
+
+// ------------------------------------------------------------------------------------------------ RMS norm of column slices
+// out [T, N] = x / sqrt(mean(x^2) + eps) * w for rows x of stride ld (a column slice of a fused projection).
+// grid (T), 256 threads.
+template <typename T>
+__global__ void __launch_bounds__(256)
+rmsnorm_rows_kernel(const T* __restrict__ x, int ld, const float* __restrict__ w, T* __restrict__ out, int N,
+                    float eps) {
+  __shared__ float red[16];
+  const T* xr = x + (size_t)blockIdx.x * ld;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < N; i += 256) {
+    const float v = ldg(xr + i);
+    ss = fmaf(v, v, ss);
+  }
+  ss = block_sum(ss, red);
+  const float r = 1.f / sqrtf(ss / (float)N + eps);
+  for (int i = threadIdx.x; i < N; i += 256) stg(out + (size_t)blockIdx.x * N + i, ldg(xr + i) * r * w[i]);
+}
+
+// ------------------------------------------------------------------------------------------------ q / k norm + store
+// proj [T, ld]: q heads at column qoff (H x d), k heads at koff (G x d).  q_out [T, H, d] = q / rms(q) * qw;
+// k_cache [nblk, G, BS, d] <- k / rms(k) * kw; v_cache [nblk, G, BS, d] <- k as projected (the values are the keys).
+// grid (T, ceil((H + G) / 4)), 256 threads: one wave per (token, head).
+template <typename T>
+__global__ void __launch_bounds__(256)
+qk_norm_store_kernel(const T* __restrict__ proj, int ld, int qoff, int koff, const float* __restrict__ qw,
+                     const float* __restrict__ kw, const int* __restrict__ slot_mapping, T* __restrict__ q_out,
+                     T* __restrict__ k_cache, T* __restrict__ v_cache, int H, int G, int d, int BS, long nslots,
+                     float eps) {
+  const int t = blockIdx.x, lane = threadIdx.x & 63;
+  const int u = blockIdx.y * 4 + (threadIdx.x >> 6);
+  if (u >= H + G) return;
+  const bool isq = u < H;
+  const int h = isq ? u : u - H;
+  const T* src = proj + (size_t)t * ld + (isq ? qoff : koff) + h * d;
+  float ss = 0.f;
+  for (int i = lane; i < d; i += 64) {
+    const float v = ldg(src + i);
+    ss = fmaf(v, v, ss);
+  }
+  ss = wave_sum(ss);
+  const float r = 1.f / sqrtf(ss / (float)d + eps);
+  if (isq) {
+    T* dst = q_out + ((size_t)t * H + h) * d;
+    for (int i = lane; i < d; i += 64) stg(dst + i, ldg(src + i) * r * qw[i]);
+    return;
+  }
+  const long slot = slot_mapping[t];
+  if (slot < 0) return;
+  if (!index_ok(slot, nslots, ERR_KV_SLOT)) return;
+  const size_t o = (((size_t)(slot / BS) * G + h) * BS + slot % BS) * d;
+  for (int i = lane; i < d; i += 64) {
+    const float v = ldg(src + i);
+    stg(k_cache + o + i, v * r * kw[i]);
+    v_cache[o + i] = src[i];
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ latent store
+// ckv [T, ld_c]: R latent columns, then r columns of the shared rotated key part.  k_cache [nblk, 1, BS, R + r] <-
+// latent / rms(latent) * cw | rotated part; v_cache [nblk, 1, BS, R] <- the normed latent again (the values of the
+// absorbed form).  q [T, H, R + r] (in place): the last r columns of every head are rotated.  Rotation: dim i paired
+// with i + r/2, table row p = cos[0:r/2] | sin[0:r/2] (fp32).
+// grid (T, ceil((1 + H) / 4)), 256 threads: wave 0 of a token owns the cache row, waves 1 .. H a query head each.
+template <typename T>
+__global__ void __launch_bounds__(256)
+latent_store_kernel(const T* __restrict__ ckv, int ld_c, const float* __restrict__ cw,
+                    const int* __restrict__ positions, const float* __restrict__ table, int table_rows,
+                    const int* __restrict__ slot_mapping, T* __restrict__ q, T* __restrict__ k_cache,
+                    T* __restrict__ v_cache, int H, int R, int r, int BS, long nslots, float eps) {
+  const int t = blockIdx.x, lane = threadIdx.x & 63;
+  const int u = blockIdx.y * 4 + (threadIdx.x >> 6);
+  if (u > H) return;
+  int p = positions[t];
+  if (!index_ok(p, table_rows, ERR_ROPE_POS)) p = 0;
+  const float* cs = table + (size_t)p * r;
+  const int half = r >> 1;
+  if (u > 0) {
+    T* qr = q + ((size_t)t * H + (u - 1)) * (R + r) + R;
+    for (int i = lane; i < half; i += 64) {
+      const float a = ldg(qr + i), b = ldg(qr + i + half);
+      const float c = cs[i], s = cs[half + i];
+      stg(qr + i, a * c - b * s);
+      stg(qr + i + half, b * c + a * s);
+    }
+    return;
+  }
+  const long slot = slot_mapping[t];
+  if (slot < 0) return;
+  if (!index_ok(slot, nslots, ERR_KV_SLOT)) return;
+  const T* src = ckv + (size_t)t * ld_c;
+  float ss = 0.f;
+  for (int i = lane; i < R; i += 64) {
+    const float v = ldg(src + i);
+    ss = fmaf(v, v, ss);
+  }
+  ss = wave_sum(ss);
+  const float rn = 1.f / sqrtf(ss / (float)R + eps);
+  T* kd = k_cache + (size_t)slot * (R + r);
+  T* vd = v_cache + (size_t)slot * R;
+  for (int i = lane; i < R; i += 64) {
+    const float v = ldg(src + i) * rn * cw[i];
+    stg(kd + i, v);
+    stg(vd + i, v);
+  }
+  for (int i = lane; i < half; i += 64) {
+    const float a = ldg(src + R + i), b = ldg(src + R + i + half);
+    const float c = cs[i], s = cs[half + i];
+    stg(kd + R + i, a * c - b * s);
+    stg(kd + R + i + half, b * c + a * s);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ sigmoid window attention
+// o_i = sum over keys j with 0 <= i - j < window of sigmoid(q_i . k_j * scale + bias_h) v_j: every visible key has its
+// own weight, nothing is normalised over the keys.  K and V caches [nblk, G, BS, d | vd]; q [T, H, d]; bias [H] fp32.
+// With `gate` (rows of stride gate_ld, H x vd columns) the output is multiplied by sigmoid(gate) as it is stored.
+constexpr int SW_NQ = 4;  // queries per wave (prefill)
+constexpr int SW_VC = 4;  // 64-wide value-dim chunks per lane: vd <= 256
+
+// prefill: grid (q tiles of 4 waves x SW_NQ queries, H, nseq), 256 threads.  Tiles of KT keys (K [KT][d+1], V [KT][vd],
+// fp32) are staged in LDS from the first key the tile's first query still sees; lane = key for the scores, lane =
+// value dim for the output.
+template <typename T>
+__global__ void __launch_bounds__(256)
+sigmoid_window_prefill_kernel(const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+                              T* __restrict__ out, int out_ld, const int* __restrict__ block_tables, int bt_stride,
+                              const int* __restrict__ q_start, const int* __restrict__ ctx_len,
+                              const float* __restrict__ bias, int H, int G, int d, int vd, int BS, float scale,
+                              int window, int KT, int nblocks, const T* __restrict__ gate, int gate_ld) {
+  extern __shared__ float smem[];
+  const int QT = 4 * SW_NQ;
+  const int seq = blockIdx.z, h = blockIdx.y, g = h / (H / G);
+  const int qa = q_start[seq], qlen = q_start[seq + 1] - qa, ctx = ctx_len[seq];
+  const int q0 = blockIdx.x * QT;
+  if (q0 >= qlen) return;
+  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+  const int dp = d + 1;
+  float* Ks = smem;                    // [KT][d+1]
+  float* Vs = Ks + KT * dp;            // [KT][vd]
+  float* Qs = Vs + KT * vd;            // [QT][d]
+  float* Ps = Qs + QT * d;             // [4 waves][SW_NQ][64]
+  for (int idx = threadIdx.x; idx < QT * d; idx += 256) {
+    const int qi = idx / d, i = idx - qi * d;
+    const int tq = q0 + qi;
+    Qs[idx] = tq < qlen ? ldg(q + ((size_t)(qa + tq) * H + h) * d + i) : 0.f;
+  }
+  const int pos0 = ctx - qlen;  // position of the launch's first query of this sequence
+  float acc[SW_NQ][SW_VC];
+#pragma unroll
+  for (int n = 0; n < SW_NQ; ++n)
+#pragma unroll
+    for (int c = 0; c < SW_VC; ++c) acc[n][c] = 0.f;
+  const float pb = bias[h];
+  const int last_q = min(q0 + QT, qlen) - 1;
+  const int kend = min(ctx, pos0 + last_q + 1);
+  const int kbeg = max(0, pos0 + q0 - (window - 1));
+  const int* bt = block_tables + (size_t)seq * bt_stride;
+  for (int k0 = kbeg; k0 < kend; k0 += KT) {
+    __syncthreads();
+    const int kn = min(KT, kend - k0);
+    for (int idx = threadIdx.x; idx < kn * d; idx += 256) {
+      const int kk = idx / d, i = idx - kk * d;
+      const int key = k0 + kk;
+      const int blk = bt[key / BS];
+      float v = 0.f;
+      if (index_ok(blk, nblocks, ERR_BLOCK_PREFILL))
+        v = ldg(k_cache + (((size_t)blk * G + g) * BS + key % BS) * d + i);
+      Ks[kk * dp + i] = v;
+    }
+    for (int idx = threadIdx.x; idx < kn * vd; idx += 256) {
+      const int kk = idx / vd, i = idx - kk * vd;
+      const int key = k0 + kk;
+      const int blk = bt[key / BS];
+      float v = 0.f;
+      if (blk >= 0 && blk < nblocks) v = ldg(v_cache + (((size_t)blk * G + g) * BS + key % BS) * vd + i);
+      Vs[kk * vd + i] = v;
+    }
+    __syncthreads();
+    float s[SW_NQ];
+#pragma unroll
+    for (int n = 0; n < SW_NQ; ++n) s[n] = 0.f;
+    if (lane < kn) {
+      const float* kr = Ks + lane * dp;
+      const float* qr = Qs + (wid * SW_NQ) * d;
+      for (int i = 0; i < d; ++i) {
+        const float kv = kr[i];
+#pragma unroll
+        for (int n = 0; n < SW_NQ; ++n) s[n] = fmaf(qr[n * d + i], kv, s[n]);
+      }
+    }
+    float* pw = Ps + wid * SW_NQ * 64;
+#pragma unroll
+    for (int n = 0; n < SW_NQ; ++n) {
+      const int tq = q0 + wid * SW_NQ + n;
+      const int dist = pos0 + tq - (k0 + lane);
+      const bool vis = lane < kn && tq < qlen && dist >= 0 && dist < window;
+      pw[n * 64 + lane] = vis ? sigmoid_f(fmaf(s[n], scale, pb)) : 0.f;
+    }
+    // (the wave's own LDS rows: a wave-level fence is enough)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+#pragma unroll
+    for (int c = 0; c < SW_VC; ++c) {
+      const int j = lane + 64 * c;
+      if (j < vd) {
+        for (int kk = 0; kk < kn; ++kk) {
+          const float vv = Vs[kk * vd + j];
+#pragma unroll
+          for (int n = 0; n < SW_NQ; ++n) acc[n][c] = fmaf(pw[n * 64 + kk], vv, acc[n][c]);
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int n = 0; n < SW_NQ; ++n) {
+    const int tq = q0 + wid * SW_NQ + n;
+    if (tq >= qlen) continue;
+#pragma unroll
+    for (int c = 0; c < SW_VC; ++c) {
+      const int j = lane + 64 * c;
+      if (j < vd) {
+        const float gt = gate ? sigmoid_f(ldg(gate + (size_t)(qa + tq) * gate_ld + h * vd + j)) : 1.f;
+        stg(out + (size_t)(qa + tq) * out_ld + h * vd + j, acc[n][c] * gt);
+      }
+    }
+  }
+}
+
+// decode (one query token per sequence, at position ctx - 1): grid (H, nseq), 256 threads.  The window's keys are cut
+// into 64-key tiles; each of the 4 waves takes every 4th tile (lane = key for the score, lane = value dim for the
+// output) and the waves' sums are added through LDS.
+template <typename T>
+__global__ void __launch_bounds__(256)
+sigmoid_window_decode_kernel(const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+                             T* __restrict__ out, int out_ld, const int* __restrict__ block_tables, int bt_stride,
+                             const int* __restrict__ ctx_len, const float* __restrict__ bias, int H, int G, int d,
+                             int vd, int BS, float scale, int window, int nblocks, const T* __restrict__ gate,
+                             int gate_ld) {
+  extern __shared__ float smem[];
+  const int seq = blockIdx.y, h = blockIdx.x, g = h / (H / G);
+  const int ctx = ctx_len[seq];
+  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+  float* Qs = smem;          // [d]
+  float* Ps = Qs + d;        // [4][64]
+  float* As = Ps + 4 * 64;   // [4][vd]
+  for (int i = threadIdx.x; i < d; i += 256) Qs[i] = ldg(q + ((size_t)seq * H + h) * d + i);
+  __syncthreads();
+  float acc[SW_VC];
+#pragma unroll
+  for (int c = 0; c < SW_VC; ++c) acc[c] = 0.f;
+  const float pb = bias[h];
+  const int* bt = block_tables + (size_t)seq * bt_stride;
+  float* pw = Ps + wid * 64;
+  const int kbeg = max(0, ctx - window);
+  const int ntiles = (ctx - kbeg + 63) >> 6;
+  for (int t = wid; t < ntiles; t += 4) {
+    const int key = kbeg + t * 64 + lane;
+    const bool vis = key < ctx;
+    float s = 0.f;
+    if (vis) {
+      int blk = bt[key / BS];
+      if (!index_ok(blk, nblocks, ERR_BLOCK_DECODE)) blk = 0;
+      const T* kr = k_cache + (((size_t)blk * G + g) * BS + key % BS) * d;
+      for (int i = 0; i < d; ++i) s = fmaf(Qs[i], ldg(kr + i), s);
+    }
+    pw[lane] = vis ? sigmoid_f(fmaf(s, scale, pb)) : 0.f;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    const int kn = min(64, ctx - (kbeg + t * 64));
+#pragma unroll
+    for (int c = 0; c < SW_VC; ++c) {
+      const int j = lane + 64 * c;
+      if (j < vd) {
+        float a = acc[c];
+        for (int kk = 0; kk < kn; ++kk) {
+          const int key2 = kbeg + t * 64 + kk;
+          int b2 = bt[key2 / BS];
+          if (b2 < 0 || b2 >= nblocks) b2 = 0;
+          a = fmaf(pw[kk], ldg(v_cache + (((size_t)b2 * G + g) * BS + key2 % BS) * vd + j), a);
+        }
+        acc[c] = a;
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+#pragma unroll
+  for (int c = 0; c < SW_VC; ++c) {
+    const int j = lane + 64 * c;
+    if (j < vd) As[wid * vd + j] = acc[c];
+  }
+  __syncthreads();
+  for (int j = threadIdx.x; j < vd; j += 256) {
+    const float gt = gate ? sigmoid_f(ldg(gate + (size_t)seq * gate_ld + h * vd + j)) : 1.f;
+    stg(out + (size_t)seq * out_ld + h * vd + j, ((As[j] + As[vd + j]) + (As[2 * vd + j] + As[3 * vd + j])) * gt);
+  }
+}
+
+}  // namespace grag
+
+using namespace grag;
+
+#define DT_DISPATCH(dt, ...)                   \
+  if ((dt) == 0) {                             \
+    using T = bf16;                            \
+    __VA_ARGS__                                \
+  } else {                                     \
+    using T = float;                           \
+    __VA_ARGS__                                \
+  }
+
+GRAG_API int grag_hyper_max_streams() { return HC_MAX; }
+
+GRAG_API hipError_t grag_hyper_mix(float* streams, int S, const void* y, const float* mix, const float* outc,
+                                   const float* inc, const float* w, float eps, void* out, float* out_sum, int T_,
+                                   int H, int dt, hipStream_t st) {
+  if (T_ <= 0) return hipSuccess;
+  if (S < 1 || S > HC_MAX || H > 36 * 1024) return hipErrorInvalidValue;
+  if (y != nullptr && (mix == nullptr || outc == nullptr)) return hipErrorInvalidValue;
+  if (out != nullptr && (inc == nullptr || w == nullptr)) return hipErrorInvalidValue;
+  const size_t bytes = (size_t)H * sizeof(float);
+  DT_DISPATCH(dt, {
+    if (bytes > 48 * 1024) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&hyper_mix_kernel<T>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+      if (e != hipSuccess) return e;
+    }
+    hipLaunchKernelGGL(hyper_mix_kernel<T>, dim3(T_), dim3(256), bytes, st, streams, (size_t)T_ * H, S,
+                                     (const T*)y, mix, outc, inc, w, eps, (T*)out, out_sum, H);
+  })
+  return hipGetLastError();
+}
+
+GRAG_API hipError_t grag_rmsnorm_rows(const void* x, int ld, const float* w, void* out, int T_, int N, float eps,
+                                      int dt, hipStream_t st) {
+  if (T_ <= 0) return hipSuccess;
+  DT_DISPATCH(dt, hipLaunchKernelGGL(rmsnorm_rows_kernel<T>, dim3(T_), dim3(256), 0, st, (const T*)x, ld, w, (T*)out,
+                                     N, eps);)
+  return hipGetLastError();
+}
+
+GRAG_API hipError_t grag_qk_norm_store(const void* proj, int ld, int qoff, int koff, const float* qw, const float* kw,
+                                       const int* slot_mapping, void* q_out, void* k_cache, void* v_cache, int T_,
+                                       int H, int G, int d, int BS, long nslots, float eps, int dt, hipStream_t st) {
+  if (T_ <= 0) return hipSuccess;
+  if (H + G > 4 * 65535) return hipErrorInvalidValue;
+  DT_DISPATCH(dt, hipLaunchKernelGGL(qk_norm_store_kernel<T>, dim3(T_, (H + G + 3) / 4), dim3(256), 0, st,
+                                     (const T*)proj, ld, qoff, koff, qw, kw, slot_mapping, (T*)q_out, (T*)k_cache,
+                                     (T*)v_cache, H, G, d, BS, nslots, eps);)
+  return hipGetLastError();
+}
+
+GRAG_API hipError_t grag_latent_store(const void* ckv, int ld_c, const float* cw, const int* positions,
+                                      const float* table, int table_rows, const int* slot_mapping, void* q,
+                                      void* k_cache, void* v_cache, int T_, int H, int R, int r, int BS, long nslots,
+                                      float eps, int dt, hipStream_t st) {
+  if (T_ <= 0) return hipSuccess;
+  if (H + 1 > 4 * 65535 || (r & 1)) return hipErrorInvalidValue;
+  DT_DISPATCH(dt, hipLaunchKernelGGL(latent_store_kernel<T>, dim3(T_, (H + 4) / 4), dim3(256), 0, st, (const T*)ckv,
+                                     ld_c, cw, positions, table, table_rows, slot_mapping, (T*)q, (T*)k_cache,
+                                     (T*)v_cache, H, R, r, BS, nslots, eps);)
+  return hipGetLastError();
+}
+
+static int sw_key_tile(int d, int vd, size_t* bytes) {
+  // K [KT][d+1] + V [KT][vd] + Q [16][d] + P [4][SW_NQ][64], fp32; the largest tile of 64 / 32 / 16 keys under 144 KB
+  for (int kt = 64; kt >= 16; kt >>= 1) {
+    const size_t b = ((size_t)kt * (d + 1 + vd) + 16 * (size_t)d + 4 * SW_NQ * 64) * sizeof(float);
+    if (b <= 144 * 1024 || kt == 16) {
+      *bytes = b;
+      return kt;
+    }
+  }
+  return 16;
+}
+
+GRAG_API hipError_t grag_sigmoid_window_prefill(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                                int out_ld, const int* block_tables, int bt_stride, const int* q_start,
+                                                const int* ctx_len, const float* bias, int nseq, int max_q_len, int H,
+                                                int G, int d, int vd, int BS, float scale, int window, int nblocks,
+                                                int dt, const void* gate, int gate_ld, hipStream_t st) {
+  if (nseq <= 0 || max_q_len <= 0) return hipSuccess;
+  if (vd > 64 * SW_VC || G < 1 || H % G || window < 1) return hipErrorInvalidValue;
+  size_t bytes = 0;
+  const int KT = sw_key_tile(d, vd, &bytes);
+  if (bytes > 160 * 1024) return hipErrorInvalidValue;
+  const dim3 grid((max_q_len + 4 * SW_NQ - 1) / (4 * SW_NQ), H, nseq);
+  DT_DISPATCH(dt, {
+    if (bytes > 48 * 1024) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&sigmoid_window_prefill_kernel<T>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+      if (e != hipSuccess) return e;
+    }
+    hipLaunchKernelGGL(sigmoid_window_prefill_kernel<T>, grid, dim3(256), bytes, st, (const T*)q, (const T*)k_cache,
+                       (const T*)v_cache, (T*)out, out_ld, block_tables, bt_stride, q_start, ctx_len, bias, H, G, d,
+                       vd, BS, scale, window, KT, nblocks, (const T*)gate, gate_ld);
+  })
+  return hipGetLastError();
+}
+
+GRAG_API hipError_t grag_sigmoid_window_decode(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                               int out_ld, const int* block_tables, int bt_stride, const int* ctx_len,
+                                               const float* bias, int nseq, int H, int G, int d, int vd, int BS,
+                                               float scale, int window, int nblocks, int dt, const void* gate,
+                                               int gate_ld, hipStream_t st) {
+  if (nseq <= 0) return hipSuccess;
+  if (vd > 64 * SW_VC || G < 1 || H % G || window < 1) return hipErrorInvalidValue;
+  const size_t bytes = ((size_t)d + 4 * 64 + 4 * (size_t)vd) * sizeof(float);
+  DT_DISPATCH(dt, hipLaunchKernelGGL(sigmoid_window_decode_kernel<T>, dim3(H, nseq), dim3(256), bytes, st, (const T*)q,
+                                     (const T*)k_cache, (const T*)v_cache, (T*)out, out_ld, block_tables, bt_stride,
+                                     ctx_len, bias, H, G, d, vd, BS, scale, window, nblocks, (const T*)gate,
+                                     gate_ld);)
+  return hipGetLastError();
+}

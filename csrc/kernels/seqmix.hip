@@ -910,7 +910,10 @@ sink_attn_decode_kernel(const T* __restrict__ q, const T* __restrict__ k_cache, 
 }
 
 // ------------------------------------------------------------------------------------------------ decay linear attention
-// Per head: S_t = decay_h S_(t-1) + k_t v_t^T, o_t = S_t^T q_t, with q, k, v = silu(projection) and S [d, vd] fp32.
+// Per head: S_t = decay_h S_(t-1) + k_t v_t^T, o_t = S_t^T q_t, S [d, vd] fp32.  q, k, v are the projection's columns,
+// through SiLU when `act` is set; with rd > 0 the first rd dims of q and k are rotated by the token's position
+// (dim i paired with i + rd/2, table row p = cos[0:rd/2] | sin[0:rd/2]) in fp32 on the way into LDS, and k is then
+// multiplied by kscale: nothing between the projection and the recurrence is rounded to 16 bits.
 // grid (H, nseq); thread j < vd owns column j of S in registers (DMAX rows).  Tokens of the launch are walked in
 // order, TB at a time through LDS.  Serves prefill chunks (qlen tokens) and decode rows (qlen = 1) alike.
 //
@@ -929,7 +932,9 @@ decay_attn_scan_kernel(const T* __restrict__ proj, int ld, int qoff, int koff, i
                                        const float* __restrict__ decay, float* __restrict__ state,
                                        const int* __restrict__ slots, const int* __restrict__ q_start,
                                        const int* __restrict__ ctx_len, float* __restrict__ out, int H, int d, int vd,
-                                       int nslots, float* __restrict__ ws, int maxchunks) {
+                                       int nslots, float* __restrict__ ws, int maxchunks, int act,
+                                       const int* __restrict__ positions, const float* __restrict__ rope_tab, int rd,
+                                       int tab_rows, float kscale) {
   constexpr int TB = 16;
   extern __shared__ __attribute__((aligned(16))) float smem[];  // [TB][2][dp] q | k, then [TB][vd] v
   const int dp = (d + 3) & ~3;  // d rounded up to 4 (16-B rows)
@@ -964,11 +969,23 @@ decay_attn_scan_kernel(const T* __restrict__ proj, int ld, int qoff, int koff, i
       const int tt = idx / (2 * d), r = idx - tt * 2 * d;
       const int which = r / d, i = r - which * d;
       const T* row = proj + (size_t)(qa + t0 + tt) * ld + (which ? koff : qoff) + h * d;
-      smem[(tt * 2 + which) * dp + i] = silu_acc(ldf(row + i));
+      float val = ldf(row + i);
+      if (act) val = silu_acc(val);
+      if (i < rd) {
+        const int half = rd >> 1, fi = i < half ? i : i - half;
+        float other = ldf(row + (i < half ? i + half : i - half));
+        if (act) other = silu_acc(other);
+        int p = positions[qa + t0 + tt];
+        if (!index_ok(p, tab_rows, ERR_ROPE_POS)) p = 0;
+        const float c = rope_tab[(size_t)p * rd + fi], sn = rope_tab[(size_t)p * rd + half + fi];
+        val = i < half ? val * c - other * sn : val * c + other * sn;
+      }
+      smem[(tt * 2 + which) * dp + i] = which ? val * kscale : val;
     }
     for (int idx = threadIdx.x; idx < nb * vd; idx += blockDim.x) {
       const int tt = idx / vd, i = idx - tt * vd;
-      vsm[idx] = silu_acc(ldf(proj + (size_t)(qa + t0 + tt) * ld + voff + h * vd + i));
+      const float val = ldf(proj + (size_t)(qa + t0 + tt) * ld + voff + h * vd + i);
+      vsm[idx] = act ? silu_acc(val) : val;
     }
     __syncthreads();
     if (j < vd) {
@@ -1044,21 +1061,24 @@ __global__ void decay_chunk_prefix_kernel(const float* __restrict__ decay, float
   Sg[e] = S;
 }
 
-// out [T, out_ld slice] = out_scale * x / rms(x) * w * sigmoid(gate), x fp32 [T, N]; gate at proj column goff.
+// out [T, out_ld slice] = out_scale * x / rms(x) * w * gate(g), x fp32 [T, groups * N] normalised per group of N
+// columns (grid (T, groups): the whole row, or one head at a time); w may be null (no weight); g at proj column
+// goff, gate = sigmoid (silu_gate 0) or SiLU (1).
 template <typename T>
 __global__ void gated_rmsnorm_kernel(const float* __restrict__ x, const float* __restrict__ w,
                                      const T* __restrict__ proj, int ld, int goff, T* __restrict__ out, int out_ld,
-                                     int N, float eps, float out_scale) {
+                                     int N, float eps, float out_scale, int silu_gate) {
   __shared__ float red[16];
-  const int t = blockIdx.x;
-  const float* xr = x + (size_t)t * N;
+  const int t = blockIdx.x, c0 = blockIdx.y * N;
+  const float* xr = x + (size_t)t * N * gridDim.y + c0;
   float ss = 0.f;
   for (int i = threadIdx.x; i < N; i += blockDim.x) ss += xr[i] * xr[i];
   ss = block_sum(ss, red);
   const float r = out_scale / sqrtf(ss / (float)N + eps);
   for (int i = threadIdx.x; i < N; i += blockDim.x) {
-    const float gt = sigmoid_acc(ldf(proj + (size_t)t * ld + goff + i));
-    stf(out + (size_t)t * out_ld + i, xr[i] * r * w[i] * gt);
+    const float g = ldf(proj + (size_t)t * ld + goff + c0 + i);
+    const float gt = silu_gate ? silu_acc(g) : sigmoid_acc(g);
+    stf(out + (size_t)t * out_ld + c0 + i, xr[i] * r * (w ? w[c0 + i] : 1.f) * gt);
   }
 }
 
@@ -1139,20 +1159,22 @@ __global__ void mingru_chunk_kernel(const T* __restrict__ proj, int ld, int zoff
 }
 
 // ------------------------------------------------------------------------------------------------ clamped GLU
-// gu [T, 2F] (gate | up): y = g sigmoid(alpha g) (u + 1), g = min(gate, limit), u = clamp(up, -limit, limit).
+// gu [T, 2F] (gate | up): y = g sigmoid(alpha g) (u + shift), g = min(gate, limit), u = clamp(up, -limit, limit).
+// (limit = +inf, alpha = 1, shift = 0: the plain SiLU-gated unit.)
 template <typename T>
-__global__ void clamped_glu_kernel(const T* __restrict__ gu, T* __restrict__ out, int F, float limit, float alpha) {
+__global__ void clamped_glu_kernel(const T* __restrict__ gu, T* __restrict__ out, int F, float limit, float alpha,
+                                   float shift) {
   const size_t t = blockIdx.x;
   const int i = blockIdx.y * blockDim.x + threadIdx.x;
   if (i >= F) return;
   const float g = fminf(ldf(gu + t * 2 * F + i), limit);
   const float u = fminf(fmaxf(ldf(gu + t * 2 * F + F + i), -limit), limit);
-  stf(out + t * F + i, g * sigmoid_acc(alpha * g) * (u + 1.f));
+  stf(out + t * F + i, g * sigmoid_acc(alpha * g) * (u + shift));
 }
 
 // bf16, F % 8 == 0: 16-byte loads and stores, 8 elements per thread
 __global__ void clamped_glu_vec_kernel(const bf16* __restrict__ gu, bf16* __restrict__ out, int F, float limit,
-                                       float alpha) {
+                                       float alpha, float shift) {
   const size_t t = blockIdx.x;
   const int i = (blockIdx.y * blockDim.x + threadIdx.x) * 8;
   if (i >= F) return;
@@ -1163,7 +1185,7 @@ __global__ void clamped_glu_vec_kernel(const bf16* __restrict__ gu, bf16* __rest
   for (int e = 0; e < 8; ++e) {
     const float g = fminf(bits2f(g8[e]), limit);
     const float u = fminf(fmaxf(bits2f(u8[e]), -limit), limit);
-    o[e] = f2bits(g * sigmoid_acc(alpha * g) * (u + 1.f));
+    o[e] = f2bits(g * sigmoid_acc(alpha * g) * (u + shift));
   }
   *reinterpret_cast<bf16x8_t*>(out + t * F + i) = o;
 }
@@ -1332,14 +1354,16 @@ GRAG_API hipError_t grag_sink_attn_decode(const void* q, const void* k_cache, co
 template <typename T, int MODE>
 static hipError_t launch_decay_scan(const T* proj, int ld, int qoff, int koff, int voff, const float* decay,
                                     float* state, const int* slots, const int* q_start, const int* ctx_len, float* out,
-                                    int nseq, int H, int d, int vd, int nslots, float* ws, int maxchunks,
+                                    int nseq, int H, int d, int vd, int nslots, float* ws, int maxchunks, int act,
+                                    const int* positions, const float* rope_tab, int rd, int tab_rows, float kscale,
                                     hipStream_t st) {
   const int threads = ((vd + 63) / 64) * 64;
   const size_t bytes = (size_t)16 * (2 * ((d + 3) & ~3) + vd) * sizeof(float);
   const dim3 grid(H, nseq, MODE == 0 ? 1 : maxchunks);
 #define DECAY_LAUNCH(DM)                                                                                     \
   hipLaunchKernelGGL((decay_attn_scan_kernel<T, DM, MODE>), grid, dim3(threads), bytes, st, proj, ld, qoff, koff, \
-                     voff, decay, state, slots, q_start, ctx_len, out, H, d, vd, nslots, ws, maxchunks)
+                     voff, decay, state, slots, q_start, ctx_len, out, H, d, vd, nslots, ws, maxchunks, act, positions,  \
+                     rope_tab, rd, tab_rows, kscale)
   if (d <= 16) {
     DECAY_LAUNCH(16);
   } else if (d <= 32) {
@@ -1362,30 +1386,38 @@ GRAG_API int grag_decay_attn_chunk() { return DECAY_CHUNK; }
 GRAG_API hipError_t grag_decay_attn_scan(const void* proj, int ld, int qoff, int koff, int voff, const float* decay,
                                          float* state, const int* slots, const int* q_start, const int* ctx_len,
                                          float* out, int nseq, int H, int d, int vd, int nslots, int dt, float* ws,
-                                         int max_q_len, hipStream_t st) {
+                                         int max_q_len, int act, const int* positions, const float* rope_tab, int rd,
+                                         int tab_rows, float kscale, hipStream_t st) {
   if (nseq <= 0) return hipSuccess;
   if (d > 256 || vd > 256) return hipErrorInvalidValue;
+  if (rd < 0 || rd > d || (rd & 1) || (rd > 0 && (positions == nullptr || rope_tab == nullptr))) return hipErrorInvalidValue;
   if (ws == nullptr || max_q_len <= DECAY_CHUNK) {
     DT_DISPATCH(dt, return (launch_decay_scan<T, 0>((const T*)proj, ld, qoff, koff, voff, decay, state, slots, q_start,
-                                                    ctx_len, out, nseq, H, d, vd, nslots, nullptr, 0, st));)
+                                                    ctx_len, out, nseq, H, d, vd, nslots, nullptr, 0, act, positions, rope_tab,
+                                                    rd, tab_rows, kscale, st));)
   }
   const int maxchunks = (max_q_len + DECAY_CHUNK - 1) / DECAY_CHUNK;
   hipError_t e;
   DT_DISPATCH(dt, e = (launch_decay_scan<T, 1>((const T*)proj, ld, qoff, koff, voff, decay, state, slots, q_start,
-                                               ctx_len, out, nseq, H, d, vd, nslots, ws, maxchunks, st));)
+                                               ctx_len, out, nseq, H, d, vd, nslots, ws, maxchunks, act, positions, rope_tab,
+                                               rd, tab_rows, kscale, st));)
   if (e != hipSuccess) return e;
   hipLaunchKernelGGL(decay_chunk_prefix_kernel, dim3(H, nseq, (d * vd + 255) / 256), dim3(256), 0, st, decay, state, slots, q_start, ctx_len,
                      ws, maxchunks, H, d, vd, nslots);
   DT_DISPATCH(dt, e = (launch_decay_scan<T, 2>((const T*)proj, ld, qoff, koff, voff, decay, state, slots, q_start,
-                                               ctx_len, out, nseq, H, d, vd, nslots, ws, maxchunks, st));)
+                                               ctx_len, out, nseq, H, d, vd, nslots, ws, maxchunks, act, positions, rope_tab,
+                                               rd, tab_rows, kscale, st));)
   return e;
 }
 
 GRAG_API hipError_t grag_gated_rmsnorm(const float* x, const float* w, const void* proj, int ld, int goff, void* out,
-                                       int out_ld, int T_, int N, float eps, float out_scale, int dt, hipStream_t st) {
+                                       int out_ld, int T_, int N, float eps, float out_scale, int dt, int groups,
+                                       int silu_gate, hipStream_t st) {
   if (T_ <= 0) return hipSuccess;
-  DT_DISPATCH(dt, hipLaunchKernelGGL(gated_rmsnorm_kernel<T>, dim3(T_), dim3(256), 0, st, x, w, (const T*)proj, ld,
-                                     goff, (T*)out, out_ld, N, eps, out_scale);)
+  if (groups < 1 || groups > 65535 || N % groups) return hipErrorInvalidValue;
+  const int threads = N / groups <= 64 ? 64 : N / groups <= 128 ? 128 : 256;
+  DT_DISPATCH(dt, hipLaunchKernelGGL(gated_rmsnorm_kernel<T>, dim3(T_, groups), dim3(threads), 0, st, x, w,
+                                     (const T*)proj, ld, goff, (T*)out, out_ld, N / groups, eps, out_scale, silu_gate);)
   return hipGetLastError();
 }
 
@@ -1416,15 +1448,15 @@ GRAG_API hipError_t grag_mingru_scan(const void* proj, int ld, int zoff, int xof
 }
 
 GRAG_API hipError_t grag_clamped_glu(const void* gu, void* out, int T_, int F, float limit, float alpha, int dt,
-                                     hipStream_t st) {
+                                     float shift, hipStream_t st) {
   if (T_ <= 0) return hipSuccess;
   if (dt == 0 && F % 8 == 0 && (reinterpret_cast<uintptr_t>(gu) & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0) {
     hipLaunchKernelGGL(clamped_glu_vec_kernel, dim3(T_, (F / 8 + 255) / 256), dim3(256), 0, st, (const bf16*)gu,
-                       (bf16*)out, F, limit, alpha);
+                       (bf16*)out, F, limit, alpha, shift);
     return hipGetLastError();
   }
   const dim3 grid(T_, (F + 255) / 256);
   DT_DISPATCH(dt, hipLaunchKernelGGL(clamped_glu_kernel<T>, grid, dim3(256), 0, st, (const T*)gu, (T*)out, F, limit,
-                                     alpha);)
+                                     alpha, shift);)
   return hipGetLastError();
 }

@@ -14,6 +14,10 @@ def build_decoder(cfg, **kw):
         from .zofesun import ZofesunModel
 
         return ZofesunModel(cfg, **kw)
+    if cfg.arch == "namudra":
+        from .namudra import NamudraModel
+
+        return NamudraModel(cfg, **kw)
     from .qwen2 import Qwen2Model
 
     return Qwen2Model(cfg, **kw)

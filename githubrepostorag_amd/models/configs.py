@@ -100,20 +100,59 @@ class DecayAttnSpec:
 
 
 @dataclass(frozen=True)
+class RetentionSpec:
+    """Linear attention with a fixed decay per head (no softmax, no denominator), rotary on q and k, keys scaled
+    by dim^-1/2, every head's output divided by its RMS and gated by a SiLU projection."""
+    heads: int
+    dim: int
+    vdim: int
+    decay: tuple
+    rot_dims: int
+    rot_base: float
+
+
+@dataclass(frozen=True)
+class WindowAttnSpec:
+    """Sliding-window attention with sigmoid weights: the values are the un-normed keys, q and k are RMS-normed per
+    head, a per-head bias is added to the score, the heads are gated by a sigmoid projection."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    window: int
+
+
+@dataclass(frozen=True)
+class LatentAttnSpec:
+    """Causal softmax attention over a cached latent (kv_rank) and one rotated key part (rot_dim) shared by the
+    heads; queries through a latent of q_rank (0: read from the weight's shape)."""
+    heads: int
+    dim: int
+    rot_dim: int
+    vdim: int
+    kv_rank: int
+    q_rank: int
+    scale: float
+    rot_base: float
+
+
+@dataclass(frozen=True)
 class MixerSpec:
-    kind: str  # "parallel" | "mingru"
+    kind: str  # "parallel" | "mingru" | "retention" | "attention" | "latent_attention"
     left: SinkAttnSpec | None = None
     right: DecayAttnSpec | None = None
     left_scale: float = 1.0
     right_scale: float = 1.0
     width: int = 0  # mingru state width
+    spec: RetentionSpec | WindowAttnSpec | LatentAttnSpec | None = None  # the single-mixer kinds
 
 
 @dataclass(frozen=True)
 class GLUSpec:
     kind: str  # "dense"
     ff: int
-    limit: float
+    limit: float | None  # clamp of the gate / up branches (None: the plain SiLU-gated unit)
 
 
 @dataclass(frozen=True)
@@ -135,6 +174,7 @@ class HybridConfig:
     arch: str = "zofesun"
     max_position: int = 1 << 20  # the design has no position limit of its own: the engine's max_model_len bounds it
     tie_word_embeddings: bool = False
+    streams: int = 1  # residual streams (hyper-connections); 1 = the plain residual sum
 
     @property
     def num_layers(self) -> int:
@@ -157,6 +197,23 @@ class HybridConfig:
 
     def param_count(self) -> int:
         H = self.hidden_size
+        if self.arch == "namudra":
+            S = self.streams
+            n = 2 * self.vocab_size * H + H
+            for L in self.layers:
+                m, a = L.mixer.kind, L.mixer.spec
+                n += (1 if L.mlp is None else 2) * (H + (2 * S + S * S if S > 1 else 0))
+                if m == "retention":
+                    n += H * a.heads * (2 * a.dim + 2 * a.vdim) + a.heads * a.vdim * H
+                elif m == "attention":
+                    n += H * (2 * a.heads + a.kv_heads) * a.dim + 2 * a.dim + a.heads + a.heads * a.vdim * H
+                else:
+                    n += H * a.q_rank + a.q_rank + a.q_rank * a.heads * (a.dim + a.rot_dim)
+                    n += H * (a.kv_rank + a.rot_dim) + a.kv_rank + a.kv_rank * a.heads * (a.dim + a.vdim)
+                    n += a.heads * a.vdim * H
+                if L.mlp is not None:
+                    n += 3 * H * L.mlp.ff
+            return n
         n = 2 * self.vocab_size * H + 2 * H + 1 + self.loop_times * H
         for L in self.layers:
             n += 4 * (2 * H + 1)
@@ -226,6 +283,89 @@ def hybrid_config_to_dict(cfg: HybridConfig) -> dict:
             "loop": {"start": cfg.loop_start, "stop": cfg.loop_stop, "times": cfg.loop_times}}
 
 
+def _glu_from_dict(f):
+    if f is None:
+        return None
+    if f.get("kind", "dense") != "dense":
+        raise ValueError(f"unknown feed-forward kind {f.get('kind')!r}")
+    return GLUSpec("dense", int(f["ff"]), float(f["limit"]) if f.get("limit") is not None else None)
+
+
+def namudra_config_from_dict(d: dict, name: str = "namudra") -> HybridConfig:
+    """The Namudra design's config.json: a layer list of "retention" / "attention" / "latent_attention" mixers, each
+    with an optional dense feed-forward; ``streams`` residual streams; an optional loop.  Every size and constant
+    is read from it."""
+    layers = []
+    for e in d["layers"]:
+        kind, m = e["type"], e["mixer"]
+        if kind == "retention":
+            rot = m.get("rot") or {"dims": 0, "base": 1.0}
+            a = RetentionSpec(int(m["heads"]), int(m["dim"]), int(m["vdim"]), tuple(float(x) for x in m["decay"]),
+                              int(rot["dims"]), float(rot.get("base", 1.0)))
+            if len(a.decay) != a.heads or a.rot_dims % 2 or a.rot_dims > a.dim:
+                raise ValueError(f"bad retention sizes {m}")
+        elif kind == "attention":
+            a = WindowAttnSpec(int(m["heads"]), int(m.get("kv_heads", m["heads"])), int(m["dim"]),
+                               int(m.get("vdim", m["dim"])), float(m["scale"]), int(m["mask"]["size"]))
+            if a.heads % a.kv_heads or a.vdim != a.dim or a.window < 1:
+                raise ValueError(f"bad attention sizes {m} (the values are the keys: vdim == dim)")
+        elif kind == "latent_attention":
+            rot = m.get("rot") or {}
+            a = LatentAttnSpec(int(m["heads"]), int(m["dim"]), int(m["rot_dim"]), int(m["vdim"]), int(m["kv_rank"]),
+                               int(m.get("q_rank", 0)), float(m["scale"]), float(rot.get("base", 10000.0)))
+            if a.rot_dim % 2 or int(rot.get("dims", a.rot_dim)) != a.rot_dim:
+                raise ValueError(f"bad latent attention sizes {m} (the rotated part is rotated whole)")
+        else:
+            raise ValueError(f"unknown mixer type {kind!r}")
+        layers.append(HybridLayerSpec(MixerSpec(kind, spec=a), _glu_from_dict(e.get("mlp"))))
+    loop = d.get("loop") or {}
+    return HybridConfig(name, int(d["vocab"]), int(d["width"]), float(d["norm"]["eps"]), tuple(layers),
+                        int(loop.get("start", 0)), int(loop.get("stop", 0)), int(loop.get("times", 1)),
+                        arch="namudra", streams=int(d.get("streams", 1)))
+
+
+def namudra_config_to_dict(cfg: HybridConfig) -> dict:
+    """Back to the config.json form (checkpoint export, tests)."""
+    layers = []
+    for L in cfg.layers:
+        a, kind = L.mixer.spec, L.mixer.kind
+        if kind == "retention":
+            m = {"heads": a.heads, "dim": a.dim, "vdim": a.vdim, "decay": list(a.decay),
+                 "rot": {"dims": a.rot_dims, "base": a.rot_base}}
+        elif kind == "attention":
+            m = {"heads": a.heads, "kv_heads": a.kv_heads, "dim": a.dim, "vdim": a.vdim, "scale": a.scale,
+                 "mask": {"size": a.window}}
+        else:
+            m = {"heads": a.heads, "dim": a.dim, "rot_dim": a.rot_dim, "vdim": a.vdim, "kv_rank": a.kv_rank,
+                 "q_rank": a.q_rank, "scale": a.scale, "rot": {"dims": a.rot_dim, "base": a.rot_base}}
+        mlp = None if L.mlp is None else {"kind": L.mlp.kind, "ff": L.mlp.ff}
+        layers.append({"type": kind, "mixer": m, "mlp": mlp})
+    return {"architecture": "Namudra", "vocab": cfg.vocab_size, "width": cfg.hidden_size, "streams": cfg.streams,
+            "norm": {"eps": cfg.norm_eps}, "layers": layers,
+            "loop": {"start": cfg.loop_start, "stop": cfg.loop_stop, "times": cfg.loop_times}}
+
+
+def namudra_config(name: str, vocab: int, width: int, pattern: str, *, heads: int, kv_heads: int, dim: int, ff: int,
+                   window: int = 1024, ret_heads: int | None = None, ret_dim: int | None = None,
+                   ret_vdim: int | None = None, kv_rank: int = 256, q_rank: int = 384, rot_dim: int = 32,
+                   streams: int = 2, loop=(0, 0, 1), eps: float = 1e-6, ret_ff: bool = False) -> HybridConfig:
+    """A regular Namudra stack for benches and plumbing tests.  ``pattern``: one letter per layer, r = retention,
+    a = windowed sigmoid attention, l = latent attention; attention layers carry a feed-forward of ``ff``."""
+    rh, rdm, rvd = ret_heads or heads, ret_dim or dim, ret_vdim or dim
+    decay = tuple(1.0 - 2.0 ** (-4.0 - 6.0 * i / max(1, rh - 1)) for i in range(rh))
+    glu = GLUSpec("dense", ff, None)
+    kinds = {
+        "r": HybridLayerSpec(MixerSpec("retention", spec=RetentionSpec(rh, rdm, rvd, decay, rdm, 1e6)),
+                             glu if ret_ff else None),
+        "a": HybridLayerSpec(MixerSpec("attention", spec=WindowAttnSpec(heads, kv_heads, dim, dim, dim ** -0.5, window)),
+                             glu),
+        "l": HybridLayerSpec(MixerSpec("latent_attention", spec=LatentAttnSpec(
+            heads, dim, rot_dim, dim, kv_rank, q_rank, (dim + rot_dim) ** -0.5, 1e4)), glu),
+    }
+    return HybridConfig(name, vocab, width, eps, tuple(kinds[c] for c in pattern), *loop, arch="namudra",
+                        streams=streams)
+
+
 def zofesun_config(name: str, vocab: int, width: int, n_layers: int, *, heads: int, kv_heads: int, dim: int,
                    vdim: int, lin_heads: int, lin_dim: int, lin_vdim: int, ff: int, mingru_every: int = 0,
                    rot_dims: int | None = None, rot_base: float = 10000.0, loop=(0, 0, 1), limit: float = 7.0,
@@ -249,6 +389,14 @@ HYBRIDS = {
                                  lin_heads=12, lin_dim=128, lin_vdim=128, ff=8960, mingru_every=4),
     "zofesun-7b": zofesun_config("zofesun-7b", 32768, 3584, 4, heads=28, kv_heads=4, dim=128, vdim=128,
                                  lin_heads=28, lin_dim=128, lin_vdim=128, ff=18944, mingru_every=4),
+    # Namudra: a plumbing-test size and two bench sizes with the layer shapes of a 1.5B / 7B decoder
+    "namudra-tiny": namudra_config("namudra-tiny", 320, 96, "ralr", heads=4, kv_heads=2, dim=16, ff=160, window=9,
+                                   ret_heads=3, ret_dim=8, ret_vdim=24, kv_rank=32, q_rank=24, rot_dim=8, streams=2,
+                                   loop=(1, 3, 2)),
+    "namudra-1b": namudra_config("namudra-1b", 32768, 1536, "ralarala", heads=12, kv_heads=2, dim=128, ff=8960,
+                                 window=1024, kv_rank=192, q_rank=384, rot_dim=64, ret_ff=True),
+    "namudra-7b": namudra_config("namudra-7b", 32768, 3584, "rala", heads=28, kv_heads=4, dim=128, ff=18944,
+                                 window=1024, kv_rank=192, q_rank=768, rot_dim=64, ret_ff=True),
 }
 
 
@@ -259,6 +407,8 @@ def config_from_dir(path) -> DecoderConfig | HybridConfig:
     arch = str(d.get("architecture", "")).lower()
     if arch == "zofesun":
         return hybrid_config_from_dict(d, Path(path).name or "zofesun")
+    if arch == "namudra":
+        return namudra_config_from_dict(d, Path(path).name or "namudra")
     mt = str(d.get("model_type", "")).lower()
     if mt == "gpt2":
         return DecoderConfig(Path(path).name, d["vocab_size"], d["n_embd"], d.get("n_inner") or 4 * d["n_embd"],

@@ -84,12 +84,19 @@ _SIGS = {
     "grag_rope_vnorm_store": [P, I, I, I, I, P, P, I, P, P, P, P, I, I, I, I, I, I, I, ctypes.c_long, F, I, P],
     "grag_sink_attn_prefill": [P, P, P, P, I, P, I, P, P, P, I, I, I, I, I, I, I, F, F, I, I, P],
     "grag_sink_attn_decode": [P, P, P, P, I, P, I, P, P, I, I, I, I, I, I, F, F, I, I, I, I, P, P, P],
-    "grag_decay_attn_scan": [P, I, I, I, I, P, P, P, P, P, P, I, I, I, I, I, I, P, I, P],
+    "grag_decay_attn_scan": [P, I, I, I, I, P, P, P, P, P, P, I, I, I, I, I, I, P, I, I, P, P, I, I, F, P],
     "grag_decay_attn_chunk": [],
     "grag_mingru_chunk": [],
-    "grag_gated_rmsnorm": [P, P, P, I, I, P, I, I, I, F, F, I, P],
+    "grag_gated_rmsnorm": [P, P, P, I, I, P, I, I, I, F, F, I, I, I, P],
     "grag_mingru_scan": [P, I, I, I, I, P, P, P, P, P, P, P, I, I, I, I, P, I, P],
-    "grag_clamped_glu": [P, P, I, I, F, F, I, P],
+    "grag_clamped_glu": [P, P, I, I, F, F, I, F, P],
+    "grag_hyper_max_streams": [],
+    "grag_hyper_mix": [P, I, P, P, P, P, P, F, P, P, I, I, I, P],
+    "grag_qk_norm_store": [P, I, I, I, P, P, P, P, P, P, I, I, I, I, I, ctypes.c_long, F, I, P],
+    "grag_latent_store": [P, I, P, P, P, I, P, P, P, P, I, I, I, I, I, ctypes.c_long, F, I, P],
+    "grag_sigmoid_window_prefill": [P, P, P, P, I, P, I, P, P, P, I, I, I, I, I, I, I, F, I, I, I, P, I, P],
+    "grag_sigmoid_window_decode": [P, P, P, P, I, P, I, P, P, I, I, I, I, I, I, F, I, I, I, P, I, P],
+    "grag_rmsnorm_rows": [P, I, P, P, I, I, F, I, P],
     "grag_attn_decode_xcd": [I],
 }
 
@@ -157,7 +164,7 @@ def call(name: str, *args) -> None:
 
 
 # ---------------------------------------------------------------- device index guard (csrc/kernels/common.h)
-ERR_UNITS = ("norm", "elementwise", "attention", "gemm_tile", "gemm_stream", "seqmix")
+ERR_UNITS = ("norm", "elementwise", "attention", "gemm_tile", "gemm_stream", "seqmix", "gatedmix")
 ERR_CODES = {1 << 0: "embed_gather: token id >= vocab", 1 << 1: "qkv_rope_kvstore: KV slot id >= cache slots",
              1 << 2: "qkv_rope_kvstore: position >= RoPE table rows",
              1 << 3: "prefill attention: block-table entry >= KV blocks",

@@ -438,11 +438,27 @@ def sink_attention_ref(q, k_cache, v_cache, meta: AttnMetadata, scale: float, si
     return out
 
 
+NO_SINK = -1.0e30  # a sink logit this low adds exactly 0 to the denominator once any key is seen: plain softmax
+_no_sinks: dict = {}
+
+
+def no_sinks(H: int, device) -> torch.Tensor:
+    """[H] fp32 sink logits that switch the sink term off (cached per device and head count)."""
+    key = (H, str(device))
+    t = _no_sinks.get(key)
+    if t is None:
+        t = _no_sinks[key] = torch.full((H,), NO_SINK, dtype=torch.float32, device=device)
+    return t
+
+
 def sink_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, meta: AttnMetadata, scale: float,
-                   sinks: torch.Tensor, out: torch.Tensor | None = None, out_scale: float = 1.0) -> torch.Tensor:
+                   sinks: torch.Tensor | None, out: torch.Tensor | None = None, out_scale: float = 1.0) -> torch.Tensor:
     """Paged causal attention with a sink term, key size != value size allowed: q [T, H, d] -> out [T, H*vd]
     (``out`` may be a column slice of a wider buffer), multiplied by ``out_scale``.  Prefill chunks run the
-    tiled kernel, decode rows (one query per sequence) the decode kernel; a mixed step runs both."""
+    tiled kernel, decode rows (one query per sequence) the decode kernel; a mixed step runs both.  ``sinks``
+    None: ordinary softmax attention (the running maximum starts at NO_SINK, whose weight underflows to 0)."""
+    if sinks is None:
+        sinks = no_sinks(q.shape[1], q.device)
     T, H, d = q.shape
     G, BS, vd = v_cache.shape[1], v_cache.shape[2], v_cache.shape[3]
     if out is None:
@@ -478,4 +494,75 @@ def sink_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
         call("grag_sink_attn_prefill", ptr(q), ptr(k_cache), ptr(v_cache), ptr(out), out.stride(0),
              ptr(meta.block_tables), meta.block_tables.stride(0), ptr(meta.q_start), ptr(meta.ctx_len), ptr(sinks),
              meta.num_seqs, meta.max_q_len, H, G, d, vd, BS, float(scale), float(out_scale), k_cache.shape[0], dt)
+    return out
+
+
+# ---------------------------------------------------------------------------------------------- sigmoid window attention
+def sigmoid_window_attention_ref(q, k_cache, v_cache, meta: AttnMetadata, scale: float, bias: torch.Tensor,
+                                 window: int):
+    """fp32: q [T, H, d], caches [blocks, G, BS, d | vd] -> [T, H, vd].  Query at position i weighs every key j with
+    0 <= i - j < window by sigmoid(q . k * scale + bias[h]); the weights are not normalised over the keys."""
+    T, H, d = q.shape
+    G, BS, vd = v_cache.shape[1], v_cache.shape[2], v_cache.shape[3]
+    R = H // G
+    out = torch.zeros(T, H, vd, dtype=torch.float32, device=q.device)
+    qs, cl = meta.q_start.tolist(), meta.ctx_len.tolist()
+    for s in range(meta.num_seqs):
+        a, b = qs[s], qs[s + 1]
+        ql, ctx = b - a, cl[s]
+        if ql <= 0:
+            continue
+        lo = max(0, ctx - ql - window + 1)
+        blocks = meta.block_tables[s, : -(-ctx // BS)].long()
+        K = k_cache[blocks].permute(0, 2, 1, 3).reshape(-1, G, d)[lo:ctx].float().repeat_interleave(R, dim=1)
+        V = v_cache[blocks].permute(0, 2, 1, 3).reshape(-1, G, vd)[lo:ctx].float().repeat_interleave(R, dim=1)
+        sc = torch.einsum("phd,khd->hpk", q[a:b].float(), K) * scale + bias.float().view(H, 1, 1)
+        dist = torch.arange(ctx - ql, ctx, device=q.device)[:, None] - torch.arange(lo, ctx, device=q.device)[None, :]
+        p = torch.sigmoid(sc) * ((dist >= 0) & (dist < window))[None].float()
+        out[a:b] = torch.einsum("hpk,khd->phd", p, V)
+    return out
+
+
+def sigmoid_window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, meta: AttnMetadata,
+                             scale: float, bias: torch.Tensor, window: int, out: torch.Tensor | None = None,
+                             gate: torch.Tensor | None = None) -> torch.Tensor:
+    """Paged sliding-window attention with sigmoid weights: q [T, H, d] -> out [T, H*vd].  Prefill chunks run the
+    tiled kernel, decode rows (one query per sequence) the decode kernel; a mixed step runs both.  Only the last
+    ``window`` keys of a sequence are read.  ``gate`` [T, H*vd] (a column slice of a fused projection is fine):
+    the output is multiplied by sigmoid(gate) as it is stored."""
+    T, H, d = q.shape
+    G, BS, vd = v_cache.shape[1], v_cache.shape[2], v_cache.shape[3]
+    if out is None:
+        out = torch.empty(T, H * vd, dtype=q.dtype, device=q.device)
+    dec = meta.extra.get("decode_rows")
+    if dec is not None:
+        Tp, dmeta = dec
+        pmeta = AttnMetadata(q_start=meta.q_start, ctx_len=meta.ctx_len, block_tables=meta.block_tables,
+                             slot_mapping=meta.slot_mapping, max_q_len=meta.max_q_len, num_seqs=meta.num_seqs,
+                             num_tokens=Tp)
+        sigmoid_window_attention(q[:Tp], k_cache, v_cache, pmeta, scale, bias, window, out[:Tp],
+                                 None if gate is None else gate[:Tp])
+        sigmoid_window_attention(q[Tp:], k_cache, v_cache, dmeta, scale, bias, window, out[Tp:],
+                                 None if gate is None else gate[Tp:])
+        return out
+    if T == 0:
+        return out
+    if not q.is_cuda:
+        o = sigmoid_window_attention_ref(q, k_cache, v_cache, meta, scale, bias, window).reshape(T, H * vd)
+        out.copy_(o if gate is None else o * torch.sigmoid(gate.float()))
+        return out
+    assert q.is_contiguous() and out.stride(1) == 1 and bias.dtype == torch.float32 and bias.numel() == H
+    assert k_cache.dtype == q.dtype and v_cache.dtype == q.dtype and k_cache.shape[3] == d
+    assert gate is None or (gate.dtype == q.dtype and gate.stride(1) == 1 and gate.shape == (T, H * vd))
+    dt = 0 if q.dtype == torch.bfloat16 else 1
+    gl = 0 if gate is None else gate.stride(0)
+    if meta.is_decode and meta.max_q_len == 1:
+        call("grag_sigmoid_window_decode", ptr(q), ptr(k_cache), ptr(v_cache), ptr(out), out.stride(0),
+             ptr(meta.block_tables), meta.block_tables.stride(0), ptr(meta.ctx_len), ptr(bias), meta.num_seqs, H, G, d,
+             vd, BS, float(scale), int(window), k_cache.shape[0], dt, ptr(gate), gl)
+    else:
+        call("grag_sigmoid_window_prefill", ptr(q), ptr(k_cache), ptr(v_cache), ptr(out), out.stride(0),
+             ptr(meta.block_tables), meta.block_tables.stride(0), ptr(meta.q_start), ptr(meta.ctx_len), ptr(bias),
+             meta.num_seqs, meta.max_q_len, H, G, d, vd, BS, float(scale), int(window), k_cache.shape[0], dt,
+             ptr(gate), gl)
     return out

@@ -193,16 +193,85 @@ def rope_vnorm_store(proj: torch.Tensor, qoff: int, koff: int, voff: int, positi
     return q
 
 
-def clamped_glu(gu: torch.Tensor, limit: float, alpha: float = 1.702) -> torch.Tensor:
-    """gu [T, 2F] (gate | up) -> g sigmoid(alpha g) (u + 1) with g = min(gate, limit), u = clamp(up, +-limit)."""
+def clamped_glu(gu: torch.Tensor, limit: float | None, alpha: float = 1.702, shift: float = 1.0) -> torch.Tensor:
+    """gu [T, 2F] (gate | up) -> g sigmoid(alpha g) (u + shift) with g = min(gate, limit), u = clamp(up, +-limit);
+    ``limit`` None: no clamp.  (limit None, alpha 1, shift 0 is the plain SiLU-gated unit silu(gate) * up.)"""
     T, F2 = gu.shape
     F = F2 // 2
+    limit = math.inf if limit is None else limit
     if not gu.is_cuda:
         g = gu[:, :F].float().clamp(max=limit)
         u = gu[:, F:].float().clamp(-limit, limit)
-        return (g * torch.sigmoid(alpha * g) * (u + 1.0)).to(gu.dtype)
+        return (g * torch.sigmoid(alpha * g) * (u + shift)).to(gu.dtype)
     assert gu.is_contiguous()
     out = torch.empty(T, F, dtype=gu.dtype, device=gu.device)
     call("grag_clamped_glu", ptr(gu), ptr(out), T, F, float(limit), float(alpha),
-         0 if gu.dtype == torch.bfloat16 else 1)
+         0 if gu.dtype == torch.bfloat16 else 1, float(shift))
     return out
+
+
+# ---------------------------------------------------------------------------------------------- q / k norm + store
+def qk_norm_store(proj: torch.Tensor, qoff: int, koff: int, qw: torch.Tensor, kw: torch.Tensor,
+                  slot_mapping: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, H: int, G: int, d: int,
+                  eps: float) -> torch.Tensor:
+    """Attention whose values are its keys.  From a fused projection ``proj`` [T, ld] (q heads at column qoff, k
+    heads at koff): returns q / rms(q) * qw [T, H, d]; stores k / rms(k) * kw into k_cache and k as projected into
+    v_cache (both [blocks, G, BS, d]) at ``slot_mapping`` (-1: not stored).  The norms are per head, fp32."""
+    T = proj.shape[0]
+    BS = k_cache.shape[2]
+    if not proj.is_cuda:
+        x = proj.float()
+        q = x[:, qoff:qoff + H * d].reshape(T, H, d)
+        k = x[:, koff:koff + G * d].reshape(T, G, d)
+        qn = q / torch.sqrt(q.pow(2).mean(-1, keepdim=True) + eps) * qw.float()
+        kn = k / torch.sqrt(k.pow(2).mean(-1, keepdim=True) + eps) * kw.float()
+        ok = slot_mapping >= 0
+        sl = slot_mapping[ok].long()
+        k_cache[sl // BS, :, sl % BS] = kn[ok].to(k_cache.dtype)
+        v_cache[sl // BS, :, sl % BS] = k[ok].to(v_cache.dtype)
+        return qn.to(proj.dtype)
+    assert proj.stride(1) == 1 and k_cache.dtype == proj.dtype and v_cache.dtype == proj.dtype
+    assert k_cache.shape[1:] == (G, BS, d) and v_cache.shape == k_cache.shape and qw.numel() == d and kw.numel() == d
+    q = torch.empty(T, H, d, dtype=proj.dtype, device=proj.device)
+    call("grag_qk_norm_store", ptr(proj), proj.stride(0), qoff, koff, ptr(qw), ptr(kw), ptr(slot_mapping), ptr(q),
+         ptr(k_cache), ptr(v_cache), T, H, G, d, BS, k_cache.shape[0] * BS, float(eps),
+         0 if proj.dtype == torch.bfloat16 else 1)
+    return q
+
+
+def latent_store(ckv: torch.Tensor, cw: torch.Tensor, positions: torch.Tensor, table: torch.Tensor,
+                 slot_mapping: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                 eps: float) -> torch.Tensor:
+    """Latent attention's cache row and query rotation.  ``ckv`` [T, R + r]: a latent of R columns and r columns of
+    the key part that all heads share.  Stores latent / rms(latent) * cw | rotated part into k_cache
+    [blocks, 1, BS, R + r] and the normed latent again into v_cache [blocks, 1, BS, R] at ``slot_mapping``;
+    rotates the last r columns of every head of ``q`` [T, H, R + r] in place (``table``: rope_table of width r)."""
+    T, H = q.shape[0], q.shape[1]
+    R, BS = v_cache.shape[3], k_cache.shape[2]
+    r = k_cache.shape[3] - R
+    if not ckv.is_cuda:
+        x = ckv.float()
+        c = x[:, :R]
+        c = c / torch.sqrt(c.pow(2).mean(-1, keepdim=True) + eps) * cw.float()
+        h2 = r // 2
+        cs = table[positions.long()]
+        co, sn = cs[:, :h2], cs[:, h2:]
+
+        def rot(t, co, sn):
+            a, b = t[..., :h2], t[..., h2:]
+            return torch.cat([a * co - b * sn, b * co + a * sn], dim=-1)
+
+        kr = rot(x[:, R:], co, sn)
+        q[:, :, R:] = rot(q[:, :, R:].float(), co[:, None], sn[:, None]).to(q.dtype)
+        ok = slot_mapping >= 0
+        sl = slot_mapping[ok].long()
+        k_cache[sl // BS, 0, sl % BS] = torch.cat([c, kr], -1)[ok].to(k_cache.dtype)
+        v_cache[sl // BS, 0, sl % BS] = c[ok].to(v_cache.dtype)
+        return q
+    assert ckv.stride(1) == 1 and q.is_contiguous() and q.shape[2] == R + r and ckv.shape[1] == R + r
+    assert k_cache.dtype == ckv.dtype and v_cache.dtype == ckv.dtype and q.dtype == ckv.dtype
+    assert k_cache.shape[1] == 1 and v_cache.shape[1] == 1 and table.shape[1] == r and cw.numel() == R
+    call("grag_latent_store", ptr(ckv), ckv.stride(0), ptr(cw), ptr(positions), ptr(table), table.shape[0],
+         ptr(slot_mapping), ptr(q), ptr(k_cache), ptr(v_cache), T, H, R, r, BS, k_cache.shape[0] * BS, float(eps),
+         0 if ckv.dtype == torch.bfloat16 else 1)
+    return q

@@ -5,7 +5,7 @@ import os
 
 import torch
 
-from ._lib import call, ptr
+from ._lib import call, lib, ptr
 from .gemm import SplitKPartial
 
 
@@ -180,4 +180,48 @@ def embed_gather_f32(ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
     out = torch.empty(T, H, dtype=torch.float32, device=table.device)
     call("grag_embed_f32", ptr(ids), ptr(table), ptr(out), T, H, table.shape[0],
          0 if table.dtype == torch.bfloat16 else 1)
+    return out
+
+
+# ---------------------------------------------------------------------------------------------- hyper-connections
+def hyper_mix(streams: torch.Tensor, y: torch.Tensor | None = None, mix: torch.Tensor | None = None,
+              outc: torch.Tensor | None = None, inc: torch.Tensor | None = None, w: torch.Tensor | None = None,
+              eps: float = 1e-6, out_dtype=torch.bfloat16, want_sum: bool = False):
+    """One pass over S fp32 residual streams ``streams`` [S, T, H] (updated in place) at a sublayer boundary:
+    with ``y`` [T, H] (the sublayer's output): x_t <- sum_s mix[s, t] x_s + outc[t] y for every stream t at once;
+    then, with ``inc`` [S]: u = sum_s inc[s] x_s, returned RMS-normed as u / sqrt(mean(u^2) + eps) * w in
+    ``out_dtype`` (``w`` [H] fp32 is the norm's whole multiplier) and / or as it is in fp32 (``want_sum``).
+    Returns (normed | None, sum | None).  S = 1 with mix = outc = inc = 1 is the ordinary residual sum."""
+    assert streams.dtype == torch.float32 and streams.is_contiguous() and streams.dim() == 3
+    S, T, H = streams.shape
+    if not _on_gpu(streams):
+        if y is not None:
+            streams.copy_(torch.einsum("st,snh->tnh", mix.float(), streams) + outc.float()[:, None, None] * y.float())
+        if inc is None:
+            return None, None
+        u = torch.einsum("s,snh->nh", inc.float(), streams)
+        h = None if w is None else (u / torch.sqrt(u.pow(2).mean(-1, keepdim=True) + eps) * w.float()).to(out_dtype)
+        return h, (u if want_sum else None)
+    if S > lib().grag_hyper_max_streams():
+        raise ValueError(f"{S} residual streams: the kernel holds at most {lib().grag_hyper_max_streams()}")
+    if y is not None:
+        assert y.dtype == out_dtype and y.is_contiguous() and y.shape == (T, H)
+    out = torch.empty(T, H, dtype=out_dtype, device=streams.device) if (inc is not None and w is not None) else None
+    usum = torch.empty(T, H, dtype=torch.float32, device=streams.device) if (inc is not None and want_sum) else None
+    call("grag_hyper_mix", ptr(streams), S, ptr(y), ptr(mix), ptr(outc), ptr(inc), ptr(w), float(eps), ptr(out),
+         ptr(usum), T, H, 0 if out_dtype == torch.bfloat16 else 1)
+    return out, usum
+
+
+def rmsnorm_rows(x: torch.Tensor, w: torch.Tensor, eps: float) -> torch.Tensor:
+    """x [T, N] (rows may be a column slice of a wider tensor; bf16 or fp32) -> x / sqrt(mean(x^2) + eps) * w
+    (w fp32 [N]), contiguous, in x's dtype; the statistics are fp32."""
+    T, N = x.shape
+    if not _on_gpu(x):
+        xf = x.float()
+        return (xf / torch.sqrt(xf.pow(2).mean(-1, keepdim=True) + eps) * w.float()).to(x.dtype)
+    assert x.stride(1) == 1 and w.dtype == torch.float32 and w.numel() == N
+    out = torch.empty(T, N, dtype=x.dtype, device=x.device)
+    call("grag_rmsnorm_rows", ptr(x), x.stride(0), ptr(w), ptr(out), T, N, float(eps),
+         0 if x.dtype == torch.bfloat16 else 1)
     return out

@@ -37,39 +37,60 @@ def _parts(meta: AttnMetadata):
 
 
 def decay_attention(proj: torch.Tensor, qoff: int, koff: int, voff: int, decay: torch.Tensor, state: torch.Tensor,
-                    meta: AttnMetadata, H: int, d: int, vd: int) -> torch.Tensor:
-    """Linear attention with decay.  From the fused projection ``proj`` [T, ld]: q, k = silu(columns qoff / koff,
-    H x d), v = silu(columns voff, H x vd).  Per head S_t = decay_h S_(t-1) + k_t v_t^T (state [slots, H, d, vd]
-    fp32), o_t = S_t^T q_t.  Returns o [T, H*vd] fp32."""
+                    meta: AttnMetadata, H: int, d: int, vd: int, act: bool = True, positions: torch.Tensor | None = None,
+                    rope: torch.Tensor | None = None, k_scale: float = 1.0) -> torch.Tensor:
+    """Linear attention with decay.  From the fused projection ``proj`` [T, ld]: q, k = columns qoff / koff (H x d),
+    v = columns voff (H x vd), each through SiLU when ``act``.  With ``rope`` (a rope_table [positions, rd]) the
+    first rd dims of q and k are rotated by ``positions`` (dim i paired with i + rd/2) in fp32 inside the scan, and
+    k is multiplied by ``k_scale`` after the rotation.  Per head S_t = decay_h S_(t-1) + k_t v_t^T (state
+    [slots, H, d, vd] fp32), o_t = S_t^T q_t.  Returns o [T, H*vd] fp32."""
     T = proj.shape[0]
     out = torch.empty(T, H * vd, dtype=torch.float32, device=proj.device)
+    rd = 0 if rope is None else rope.shape[1]
+    if rd and (positions is None or positions.dtype != torch.int32 or rope.dtype != torch.float32 or rd > d or rd % 2):
+        raise ValueError("rotary needs int32 positions and an fp32 table of an even width <= the head size")
     for m, r0, r1 in _parts(meta):
         if r1 <= r0:
             continue
+        pos = positions[r0:r1] if rd else None
         if not proj.is_cuda:
-            _decay_attention_cpu(proj[r0:r1], qoff, koff, voff, decay, state, m, H, d, vd, out[r0:r1])
+            _decay_attention_cpu(proj[r0:r1], qoff, koff, voff, decay, state, m, H, d, vd, out[r0:r1], act, pos, rope,
+                                 k_scale)
             continue
         assert proj.stride(1) == 1 and state.dtype == torch.float32 and state.is_contiguous()
         x = proj[r0:r1]
         ws = _chunk_ws("decay", m, H * d * vd, proj.device)
         call("grag_decay_attn_scan", ptr(x), proj.stride(0), qoff, koff, voff, ptr(decay), ptr(state),
              ptr(m.state_slots), ptr(m.q_start), ptr(m.ctx_len), ptr(out[r0:r1]), m.num_seqs, H, d, vd,
-             state.shape[0], _dt(proj), ptr(ws), m.max_q_len)
+             state.shape[0], _dt(proj), ptr(ws), m.max_q_len, 1 if act else 0, ptr(pos), ptr(rope), rd,
+             rope.shape[0] if rd else 0, float(k_scale))
     return out
 
 
-def _decay_attention_cpu(x, qoff, koff, voff, decay, state, m, H, d, vd, out):
+def _decay_attention_cpu(x, qoff, koff, voff, decay, state, m, H, d, vd, out, act=True, pos=None, rope=None,
+                         k_scale=1.0):
     F = torch.nn.functional
     qs, cl, sl = m.q_start.tolist(), m.ctx_len.tolist(), m.state_slots.tolist()
     x = x.float()
+    f = F.silu if act else (lambda t: t)
     for s in range(m.num_seqs):
         a, b = qs[s], qs[s + 1]
         if b <= a:
             continue
         S = torch.zeros(H, d, vd) if cl[s] - (b - a) == 0 else state[sl[s]].clone()
-        q = F.silu(x[a:b, qoff:qoff + H * d]).view(-1, H, d)
-        k = F.silu(x[a:b, koff:koff + H * d]).view(-1, H, d)
-        v = F.silu(x[a:b, voff:voff + H * vd]).view(-1, H, vd)
+        q = f(x[a:b, qoff:qoff + H * d]).view(-1, H, d).clone()
+        k = f(x[a:b, koff:koff + H * d]).view(-1, H, d).clone()
+        v = f(x[a:b, voff:voff + H * vd]).view(-1, H, vd)
+        if rope is not None:
+            rd = rope.shape[1]
+            h2 = rd // 2
+            cs = rope[pos[a:b].long()]
+            c, sn = cs[:, None, :h2], cs[:, None, h2:]
+            for t in (q, k):
+                u, w = t[..., :h2].clone(), t[..., h2:rd].clone()
+                t[..., :h2] = u * c - w * sn
+                t[..., h2:rd] = w * c + u * sn
+        k = k * k_scale
         lam = decay.float().view(H, 1, 1)
         for t in range(b - a):
             S = lam * S + k[t, :, :, None] * v[t, :, None, :]
@@ -77,18 +98,24 @@ def _decay_attention_cpu(x, qoff, koff, voff, decay, state, m, H, d, vd, out):
         state[sl[s]] = S
 
 
-def gated_rmsnorm(x: torch.Tensor, w: torch.Tensor, proj: torch.Tensor, goff: int, eps: float,
-                  out: torch.Tensor, out_scale: float = 1.0) -> torch.Tensor:
-    """out = out_scale * x / rms(x) * w * sigmoid(gate): x [T, N] fp32 normalised over the whole row, the gate
-    read from columns goff.. of the fused projection; ``out`` [T, N] may be a column slice of a wider buffer."""
+def gated_rmsnorm(x: torch.Tensor, w: torch.Tensor | None, proj: torch.Tensor, goff: int, eps: float,
+                  out: torch.Tensor, out_scale: float = 1.0, groups: int = 1, gate: str = "sigmoid") -> torch.Tensor:
+    """out = out_scale * x / rms(x) * w * gate(g): x [T, N] fp32 normalised over each of ``groups`` equal column
+    groups (1: the whole row; the head count: per head), ``w`` [N] optional, g read from columns goff.. of the
+    fused projection, gate "sigmoid" or "silu"; ``out`` [T, N] may be a column slice of a wider buffer."""
     T, N = x.shape
+    if gate not in ("sigmoid", "silu") or N % groups:
+        raise ValueError("gate is 'sigmoid' or 'silu', and the groups divide the row")
     if not x.is_cuda:
-        g = torch.sigmoid(proj[:, goff:goff + N].float())
-        out.copy_((x / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + eps) * w.float() * g * out_scale))
+        g = proj[:, goff:goff + N].float()
+        g = torch.sigmoid(g) if gate == "sigmoid" else torch.nn.functional.silu(g)
+        xg = x.view(T, groups, N // groups)
+        y = (xg / torch.sqrt(xg.pow(2).mean(-1, keepdim=True) + eps)).reshape(T, N)
+        out.copy_(y * (1.0 if w is None else w.float()) * g * out_scale)
         return out
     assert x.is_contiguous() and out.stride(1) == 1 and out.dtype == proj.dtype
     call("grag_gated_rmsnorm", ptr(x), ptr(w), ptr(proj), proj.stride(0), goff, ptr(out), out.stride(0), T, N,
-         float(eps), float(out_scale), _dt(proj))
+         float(eps), float(out_scale), _dt(proj), groups, 1 if gate == "silu" else 0)
     return out
 
 
