@@ -155,3 +155,68 @@ def forward(cfg, weights, tokens, taps=None):
             taps.append(sum(xs))
     x = sum(xs)
     return norm_one_plus(x, w["final.norm"], eps) @ w["head"].T
+
+
+# ------------------------------------------------------------------------------------------------ test models
+def make_config(width=48, vocab=96, streams=2, kinds=("retention", "attention", "latent_attention"), loop=(1, 3, 2),
+                no_mlp=(0,), ff=40, eps=1e-5, ret=None, att=None, lat=None):
+    """A small config.json dict.  ``ret`` / ``att`` / ``lat`` override the mixers' sizes."""
+    r = dict(heads=2, dim=8, vdim=12, decay=[0.9, 0.99], rot={"dims": 4, "base": 100.0})
+    a = dict(heads=4, kv_heads=2, dim=8, vdim=8, scale=0.4, mask={"size": 7})
+    l = dict(heads=3, dim=8, rot_dim=4, vdim=10, kv_rank=16, q_rank=12, scale=0.3, rot={"dims": 4, "base": 50.0})
+    r.update(ret or {})
+    a.update(att or {})
+    l.update(lat or {})
+    if "rot_dim" in (lat or {}) and "rot" not in (lat or {}):
+        l["rot"] = {"dims": l["rot_dim"], "base": 50.0}
+    mix = {"retention": r, "attention": a, "latent_attention": l}
+    layers = [{"type": k, "mixer": dict(mix[k]), "mlp": None if i in no_mlp else {"kind": "dense", "ff": ff}}
+              for i, k in enumerate(kinds)]
+    return {"architecture": "Namudra", "vocab": vocab, "width": width, "streams": streams, "norm": {"eps": eps},
+            "layers": layers, "loop": {"start": loop[0], "stop": loop[1], "times": loop[2]}}
+
+
+def make_weights(cfg, seed=0, hc_tensors=True):
+    """Random weights whose values are exact in bfloat16, under the checkpoint's tensor names."""
+    g = torch.Generator().manual_seed(4242 + seed)
+    W, S = cfg["width"], cfg["streams"]
+
+    def r(*shape, s=None):
+        s = shape[-1] ** -0.5 if s is None else s
+        return (torch.randn(*shape, generator=g) * s).to(torch.bfloat16)
+
+    sd = {"embed": r(cfg["vocab"], W, s=1.0), "head": r(cfg["vocab"], W), "final.norm": r(W, s=0.2)}
+    for i, L in enumerate(cfg["layers"]):
+        p, m = f"l{i}.", L["mixer"]
+        for qi in (1, 2) if L["mlp"] is not None else (1,):
+            sd[p + f"norm{qi}"] = r(W, s=0.2)
+            if S > 1 or hc_tensors:
+                sd[p + f"hc{qi}.in"] = (1.0 / S + r(S, s=0.2).float()).to(torch.bfloat16)
+                sd[p + f"hc{qi}.out"] = (1.0 + r(S, s=0.3).float()).to(torch.bfloat16)
+                sd[p + f"hc{qi}.mix"] = (torch.eye(S) + r(S, S, s=0.2).float()).to(torch.bfloat16)
+        if L["type"] == "retention":
+            H, d, vd = m["heads"], m["dim"], m["vdim"]
+            sd.update({p + "mix.q": r(H * d, W), p + "mix.k": r(H * d, W), p + "mix.v": r(H * vd, W),
+                       p + "mix.g": r(H * vd, W), p + "mix.o": r(W, H * vd)})
+        elif L["type"] == "attention":
+            H, G, d = m["heads"], m["kv_heads"], m["dim"]
+            sd.update({p + "mix.q": r(H * d, W), p + "mix.k": r(G * d, W),
+                       p + "mix.q.norm": (1.0 + r(d, s=0.2).float()).to(torch.bfloat16),
+                       p + "mix.k.norm": (1.0 + r(d, s=0.2).float()).to(torch.bfloat16),
+                       p + "mix.pb": (r(H, s=1.0).float() - 1.0).to(torch.bfloat16),
+                       p + "mix.g": r(H * d, W), p + "mix.o": r(W, H * d)})
+        else:
+            H, d, rr, vd, R, Q = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"], m["q_rank"]
+            sd.update({p + "mix.dq": r(Q, W), p + "mix.dq.norm": (1.0 + r(Q, s=0.2).float()).to(torch.bfloat16),
+                       p + "mix.uq": r(H * (d + rr), Q), p + "mix.dkv": r(R + rr, W),
+                       p + "mix.dkv.norm": (1.0 + r(R, s=0.2).float()).to(torch.bfloat16),
+                       p + "mix.uk": r(H * d, R), p + "mix.uv": r(H * vd, R), p + "mix.o": r(W, H * vd)})
+        if L["mlp"] is not None:
+            F = L["mlp"]["ff"]
+            sd.update({p + "mlp.gate": r(F, W), p + "mlp.up": r(F, W), p + "mlp.down": r(W, F)})
+    return sd
+
+
+def logits_and_taps(cfg, sd, toks):
+    taps = []
+    return forward(cfg, sd, toks, taps), torch.stack(taps)
