@@ -8,6 +8,7 @@
 // Activations are bf16 or fp32 (dt: 0 = bf16, 1 = fp32; the caches hold the same type); streams, norms, scores and
 // attention weights are fp32 in both.
 #include "common.h"
+#include "attn_tiles.h"
 
 GRAG_ERR_UNIT(gatedmix)
 
@@ -306,6 +307,146 @@ sigmoid_window_prefill_kernel(const T* __restrict__ q, const T* __restrict__ k_c
   }
 }
 
+// prefill on the matrix cores (bf16 activations, d and vd multiples of 16): grid (tiles of 64 queries, H, nseq), 4 waves
+// of 16 queries; 64-key tiles from the first key the tile's first query still sees (K [64][d+8] row-major and V in
+// 4-key groups, staged in LDS as bf16, the next tile's loads in flight while one is computed):
+//   S^T = K Q^T      v_mfma_f32_16x16x32_bf16 (bf16 products are exact in fp32, fp32 accumulation); the C fragment
+//                    (rows = keys 4*(lane/16)+i, column = query lane%16) is the A fragment of the next product,
+//   weights in fp32  sigmoid(s * scale + bias_h) for keys inside the query's window, 0 outside; no running maximum,
+//                    no rescale: every tile just adds,
+//   O += P V         with the fp32 weights split into bf16 hi + lo parts (two products): 16 mantissa bits of every
+//                    weight reach the fp32 accumulator.
+// A wave skips tiles that lie wholly after its queries or wholly before its first query's window.
+template <int NKM, int NVM>
+__global__ void __launch_bounds__(256, NKM <= 8 && NVM <= 8 ? 3 : 2)
+sigmoid_window_prefill_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_cache,
+                                   const bf16* __restrict__ v_cache, bf16* __restrict__ out, int out_ld,
+                                   const int* __restrict__ block_tables, int bt_stride,
+                                   const int* __restrict__ q_start, const int* __restrict__ ctx_len,
+                                   const float* __restrict__ bias, int H, int G, int d, int vd, int BS, float scale,
+                                   int window, int nblocks, const bf16* __restrict__ gate, int gate_ld) {
+  constexpr int KT = 64;
+  extern __shared__ __attribute__((aligned(16))) char smem_raw[];
+  const int seq = blockIdx.z, h = blockIdx.y, g = h / (H / G);
+  const int qa = q_start[seq], qlen = q_start[seq + 1] - qa, ctx = ctx_len[seq];
+  const int q0 = blockIdx.x * 64;
+  if (q0 >= qlen) return;
+  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+  const int ql = lane & 15, quad = lane >> 4;
+  const int nk = d >> 4, nv = vd >> 4;
+  const int kstride = d + 8, vstride = vd * 4 + 8;  // vstride: one 4-key group of V
+  short* Ks = reinterpret_cast<short*>(smem_raw);  // [KT][d+8] bf16 bits
+  short* Vs = Ks + KT * kstride;                   // [16][vd][4] (+8 per group)
+  const int tq = q0 + wid * 16 + ql;               // this lane's query (a fragment column)
+  const bool q_ok = tq < qlen;
+  const int nk2 = nk >> 1;
+  bf16x8_t qf[NKM / 2];
+  bf16x4_t qt = bf16x4_t{0, 0, 0, 0};
+  const bf16* qrow = q + ((size_t)(qa + (q_ok ? tq : 0)) * H + h) * d;
+#pragma unroll
+  for (int ks = 0; ks < NKM / 2; ++ks) {
+    qf[ks] = bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
+    if (ks < nk2 && q_ok) qf[ks] = *reinterpret_cast<const bf16x8_t*>(qrow + ks * 32 + quad * 8);
+  }
+  if ((nk & 1) && q_ok) qt = *reinterpret_cast<const bf16x4_t*>(qrow + (nk - 1) * 16 + quad * 4);
+  const int pos0 = ctx - qlen;
+  const int qpos = pos0 + tq;
+  // sigmoid(x) = 1 / (1 + 2^(-x log2 e)): the score and the bias are taken to the log2 domain with one fma
+  const float LOG2E = 1.4426950408889634f;
+  const float sc2 = -scale * LOG2E, pb2 = -bias[h] * LOG2E;
+  f32x4_t acc[NVM];
+#pragma unroll
+  for (int v = 0; v < NVM; ++v) acc[v] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  const int kend = min(ctx, pos0 + min(q0 + 64, qlen));
+  const int kbeg = max(0, pos0 + q0 - (window - 1));
+  const int wave_qmin = pos0 + q0 + wid * 16;
+  const int wave_qmax = pos0 + min(q0 + wid * 16 + 15, qlen - 1);
+  const int* bt = block_tables + (size_t)seq * bt_stride;
+  bf16x8_t kreg[NKM / 2], vreg[NVM / 2];
+  RowCursor rc;
+  rc.init(kbeg + (threadIdx.x >> 2), BS);
+  {
+    const int blk = tile_block(rc, bt, kbeg + (threadIdx.x >> 2), kend, nblocks, ERR_BLOCK_PREFILL);
+    tile_load(kreg, k_cache, blk, rc.off, d, G, g, BS);
+    tile_load(vreg, v_cache, blk, rc.off, vd, G, g, BS);
+  }
+  for (int k0 = kbeg; k0 < kend; k0 += KT) {
+    __syncthreads();
+    tile_store(kreg, Ks, d, kstride);
+    tile_store_v4(vreg, Vs, vd, vstride);
+    __syncthreads();
+    if (k0 + KT < kend) {  // the next tile's loads fly while this one is computed
+      rc.advance(BS);
+      const int blk = tile_block(rc, bt, k0 + KT + (threadIdx.x >> 2), kend, nblocks, ERR_BLOCK_PREFILL);
+      tile_load(kreg, k_cache, blk, rc.off, d, G, g, BS);
+      tile_load(vreg, v_cache, blk, rc.off, vd, G, g, BS);
+    }
+    if (k0 > wave_qmax || k0 + KT - 1 < wave_qmin - (window - 1)) continue;  // no key of the tile is seen by this wave
+    f32x4_t st[4];
+#pragma unroll
+    for (int n = 0; n < 4; ++n) {
+      st[n] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      const short* kr = Ks + (16 * n + ql) * kstride;
+#pragma unroll
+      for (int ks = 0; ks < NKM / 2; ++ks) {
+        if (ks < nk2) {
+          const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(kr + ks * 32 + quad * 8);
+          st[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qf[ks], st[n], 0, 0, 0);
+        }
+      }
+      if (nk & 1) {
+        const bf16x4_t a = *reinterpret_cast<const bf16x4_t*>(kr + (nk - 1) * 16 + quad * 4);
+        st[n] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, qt, st[n], 0, 0, 0);
+      }
+    }
+    // a tile wholly inside every query's window of this wave (and inside the context) needs no mask
+    const bool interior = k0 + KT - 1 <= wave_qmin && k0 >= wave_qmax - (window - 1) && k0 + KT <= kend &&
+                          q0 + wid * 16 + 15 < qlen;
+#pragma unroll
+    for (int n = 0; n < 4; ++n)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = k0 + 16 * n + 4 * quad + i;
+        const float p = __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(fmaf(st[n][i], sc2, pb2)));
+        const bool vis = interior || (q_ok && key < kend && key <= qpos && qpos - key < window);
+        st[n][i] = vis ? p : 0.f;
+      }
+#pragma unroll
+    for (int np = 0; np < 2; ++np) {  // 32 keys per product: k-slots j < 4 are keys 32np + 4*quad + j, j >= 4 keys + 16
+      bf16x8_t ph, pl;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float p = st[2 * np + (j >> 2)][j & 3];
+        const short hi = f2bits(p);
+        ph[j] = hi;
+        pl[j] = f2bits(p - bits2f(hi));
+      }
+      const short* vr = Vs + (8 * np + quad) * vstride + ql * 4;
+#pragma unroll
+      for (int v = 0; v < NVM; ++v) {
+        if (v < nv) {
+          const bf16x4_t b0 = *reinterpret_cast<const bf16x4_t*>(vr + 64 * v);
+          const bf16x4_t b1 = *reinterpret_cast<const bf16x4_t*>(vr + 4 * vstride + 64 * v);
+          const bf16x8_t b = bf16x8_t{b0[0], b0[1], b0[2], b0[3], b1[0], b1[1], b1[2], b1[3]};
+          acc[v] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ph, b, acc[v], 0, 0, 0);
+          acc[v] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pl, b, acc[v], 0, 0, 0);
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int tr = q0 + wid * 16 + 4 * quad + i;  // the query of accumulator row i
+    if (tr < qlen) {
+      bf16* orow = out + (size_t)(qa + tr) * out_ld + h * vd + ql;
+      const bf16* grow = gate ? gate + (size_t)(qa + tr) * gate_ld + h * vd + ql : nullptr;
+#pragma unroll
+      for (int v = 0; v < NVM; ++v)
+        if (v < nv) orow[16 * v] = (bf16)(acc[v][i] * (grow ? sigmoid_f((float)grow[16 * v]) : 1.f));
+    }
+  }
+}
+
 // decode (one query token per sequence, at position ctx - 1): grid (H, nseq), 256 threads.  The window's keys are cut
 // into 64-key tiles; each of the 4 waves takes every 4th tile (lane = key for the score, lane = value dim for the
 // output) and the waves' sums are added through LDS.
@@ -461,6 +602,28 @@ GRAG_API hipError_t grag_sigmoid_window_prefill(const void* q, const void* k_cac
                                                 int dt, const void* gate, int gate_ld, hipStream_t st) {
   if (nseq <= 0 || max_q_len <= 0) return hipSuccess;
   if (vd > 64 * SW_VC || G < 1 || H % G || window < 1) return hipErrorInvalidValue;
+  if (dt == 0 && max_q_len >= 16 && d % 16 == 0 && vd % 16 == 0 && d <= 256 && vd <= 256 &&
+      (reinterpret_cast<uintptr_t>(q) & 15) == 0) {
+    const size_t mb = ((size_t)64 * (d + 8) + (size_t)16 * (vd * 4 + 8)) * sizeof(short);
+    const dim3 mgrid((max_q_len + 63) / 64, H, nseq);
+#define SW_MFMA(NK, NV)                                                                                             \
+  {                                                                                                                 \
+    if (mb > 48 * 1024) {                                                                                           \
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&sigmoid_window_prefill_mfma_kernel<NK, NV>), \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)mb);                      \
+      if (e != hipSuccess) return e;                                                                                \
+    }                                                                                                               \
+    hipLaunchKernelGGL((sigmoid_window_prefill_mfma_kernel<NK, NV>), mgrid, dim3(256), mb, st, (const bf16*)q,      \
+                       (const bf16*)k_cache, (const bf16*)v_cache, (bf16*)out, out_ld, block_tables, bt_stride,     \
+                       q_start, ctx_len, bias, H, G, d, vd, BS, scale, window, nblocks, (const bf16*)gate, gate_ld); \
+  }
+    const int nk = d / 16, nv = vd / 16;
+    if (nk <= 4 && nv <= 4) SW_MFMA(4, 4)
+    else if (nk <= 8 && nv <= 8) SW_MFMA(8, 8)
+    else SW_MFMA(16, 16)
+#undef SW_MFMA
+    return hipGetLastError();
+  }
   size_t bytes = 0;
   const int KT = sw_key_tile(d, vd, &bytes);
   if (bytes > 160 * 1024) return hipErrorInvalidValue;

@@ -1,7 +1,9 @@
-"""``bench.py --hybrid``: prefill and decode throughput of the Zofesun hybrid decoder beside the Qwen2 decoder of
-equal size (same width, heads, head size, FFN width, layer count, vocabulary; random weights, synthetic token
-ids), both through LLMEngine.generate, and a per-kernel table: each new kernel and the like kernel of Qwen2 as a
-fraction of the roofline of what bounds it (HBM bytes or matrix / vector flops)."""
+"""``bench.py --hybrid [zofesun|namudra]``: prefill and decode throughput of a hybrid decoder beside the decoders of
+equal size that the engine already serves (same width, heads, head size, FFN width, layer count, vocabulary; random
+weights, synthetic token ids), all through LLMEngine.generate, and a per-kernel table: each new kernel and the
+like kernel of the closest model as a fraction of the roofline of what bounds it (HBM bytes or matrix / vector
+flops).  Zofesun stands beside Qwen2; Namudra beside Zofesun (the closest: fp32 residual, decay scan, sink
+attention kernels) and Qwen2."""
 from __future__ import annotations
 
 import json
@@ -44,6 +46,19 @@ def _models(name, dev):
                         lin_vdim=D, ff=ff, mingru_every=every)
     qc = DecoderConfig(f"qwen2-{name}", VOCAB, W, ff, nl, H, G, D, max_position=32768)
     return (lambda: ZofesunModel(zc, device=dev, seed=1)), (lambda: Qwen2Model(qc, device=dev, seed=1))
+
+
+def _namudra_models(name, dev):
+    """Namudra at a bench size: per four layers retention, windowed sigmoid attention, latent attention, windowed
+    attention (every layer with a feed-forward, two residual streams), beside the Zofesun and Qwen2 stacks."""
+    from ..models.configs import namudra_config
+    from ..models.namudra import NamudraModel
+
+    W, H, G, D, ff, nl, _ = SIZES[name]
+    nc = namudra_config(f"namudra-{name}", VOCAB, W, ("rala" * nl)[:nl], heads=H, kv_heads=G, dim=D, ff=ff,
+                        window=1024, kv_rank=192, q_rank=W // 4, rot_dim=64, streams=2, ret_ff=True)
+    mk_z, mk_q = _models(name, dev)
+    return (lambda: NamudraModel(nc, device=dev, seed=1)), mk_z, mk_q
 
 
 def _engine_numbers(make, dev, batch, prompt_len, gen_len, graphs=True):
@@ -162,7 +177,133 @@ def _kernel_table(dev, H=28, G=4, D=128, W=3584, ff=18944, T=2048, B=64, ctx=204
     return rows
 
 
+def _namudra_kernel_table(dev, H=28, G=4, D=128, W=3584, T=2048, B=64, ctx=2048, bs=16, win=1024, R=192, r=64, S=2):
+    """[(kernel, seconds, bound, fraction of roofline)] for Namudra's kernels and the like kernels of Zofesun."""
+    from ..ops.attention import AttnMetadata, sigmoid_window_attention, sink_attention
+    from ..ops.elementwise import latent_store, qk_norm_store, rope_table, rope_vnorm_store
+    from ..ops.norm import dyt_residual, hyper_mix, rmsnorm_rows
+    from ..ops.recurrent import decay_attention, gated_rmsnorm
+
+    bf = torch.bfloat16
+    i32 = dict(dtype=torch.int32, device=dev)
+    rows = []
+
+    def add(name, sec, flops=0.0, bytes_=0.0, peak=MFMA_BF16):
+        t_c, t_m = flops / peak, bytes_ / HBM_BPS
+        rows.append({"kernel": name, "us": round(sec * 1e6, 1), "bound": "flops" if t_c >= t_m else "bytes",
+                     "roofline_fraction": round(max(t_c, t_m) / sec, 4)})
+
+    nb = T // bs
+    meta = AttnMetadata(q_start=torch.tensor([0, T], **i32), ctx_len=torch.tensor([T], **i32),
+                        block_tables=(torch.arange(nb, **i32) + 1).view(1, nb), slot_mapping=torch.arange(T, **i32) + bs,
+                        max_q_len=T, num_seqs=1, num_tokens=T, state_slots=torch.tensor([0], **i32))
+    nbd = ctx // bs
+    part_o = torch.empty(8 * B * H * max(D, R), device=dev)
+    part_ml = torch.empty(8 * B * H * 2, device=dev)
+    dmeta = AttnMetadata(q_start=torch.arange(B + 1, **i32), ctx_len=torch.full((B,), ctx, **i32),
+                         block_tables=(torch.arange(B * nbd, **i32) + 1).view(B, nbd), slot_mapping=None, max_q_len=1,
+                         num_seqs=B, num_tokens=B, is_decode=True, num_splits=8, split_len=ctx // 8, part_o=part_o,
+                         part_ml=part_ml, state_slots=torch.arange(B, **i32))
+    # ---- prefill attention, one prompt of T tokens: windowed sigmoid | latent (one kv head, key R + r, value R) | sink
+    kc = torch.randn(nb + 1, G, bs, D, device=dev).to(bf)
+    vc = torch.randn(nb + 1, G, bs, D, device=dev).to(bf)
+    q = torch.randn(T, H, D, device=dev).to(bf)
+    gate = torch.randn(T, H * D, device=dev).to(bf)
+    pb = torch.zeros(H, device=dev)
+    pairs = T * (T + 1) / 2 - (T - win) * (T - win + 1) / 2  # visible (query, key) pairs
+    add("sigmoid_window_prefill (window 1024)", _timed(lambda: sigmoid_window_attention(q, kc, vc, meta, 0.09, pb, win, gate=gate)),
+        flops=4.0 * pairs * H * D)
+    add("zofesun sink_attn_prefill", _timed(lambda: sink_attention(q, kc, vc, meta, 0.09, pb)), flops=4.0 * T * T / 2 * H * D)
+    kl = torch.randn(nb + 1, 1, bs, R + r, device=dev).to(bf)
+    vl = torch.randn(nb + 1, 1, bs, R, device=dev).to(bf)
+    ql = torch.randn(T, H, R + r, device=dev).to(bf)
+    add("latent attention prefill (sink kernel, no sink)", _timed(lambda: sink_attention(ql, kl, vl, meta, 0.06, None)),
+        flops=2.0 * T * T / 2 * H * (2 * R + r))
+    # ---- decode attention: B rows of ctx keys
+    kd = torch.randn(B * nbd + 1, G, bs, D, device=dev).to(bf)
+    vd_ = torch.randn(B * nbd + 1, G, bs, D, device=dev).to(bf)
+    qd = torch.randn(B, H, D, device=dev).to(bf)
+    gd = torch.randn(B, H * D, device=dev).to(bf)
+    add("sigmoid_window_decode (window 1024)", _timed(lambda: sigmoid_window_attention(qd, kd, vd_, dmeta, 0.09, pb, win, gate=gd)),
+        bytes_=2.0 * B * win * G * D * 2)
+    add("zofesun sink_attn_decode", _timed(lambda: sink_attention(qd, kd, vd_, dmeta, 0.09, pb)), bytes_=2.0 * B * ctx * G * D * 2)
+    kld = torch.randn(B * nbd + 1, 1, bs, R + r, device=dev).to(bf)
+    vld = torch.randn(B * nbd + 1, 1, bs, R, device=dev).to(bf)
+    qld = torch.randn(B, H, R + r, device=dev).to(bf)
+    add("latent attention decode (sink kernel, no sink)", _timed(lambda: sink_attention(qld, kld, vld, dmeta, 0.06, None)),
+        bytes_=B * ctx * (2 * R + r) * 2.0)
+    # ---- projection post-processing + cache stores
+    proj = torch.randn(T, (2 * H + G) * D, device=dev).to(bf)
+    ones = torch.ones(D, device=dev)
+    add("qk_norm_store", _timed(lambda: qk_norm_store(proj, 0, H * D, ones, ones, meta.slot_mapping, kc, vc, H, G, D, 1e-6)),
+        bytes_=T * (2 * H + 3 * G) * D * 2.0)
+    pos = torch.arange(T, **i32)
+    tab = rope_table(T, D, 1e4, dev)
+    add("zofesun rope_vnorm_store", _timed(lambda: rope_vnorm_store(proj, 0, H * D, (H + G) * D, pos, tab, meta.slot_mapping, kc, vc,
+                                                                    H, G, D, D, D, 1e-5)), bytes_=T * (H + 2 * G) * D * 2 * 2.0)
+    ckv = torch.randn(T, R + r, device=dev).to(bf)
+    tabr = rope_table(T, r, 1e4, dev)
+    add("latent_store", _timed(lambda: latent_store(ckv, torch.ones(R, device=dev), pos, tabr, meta.slot_mapping, ql, kl, vl, 1e-6)),
+        bytes_=T * ((R + r) * 2 + R + 2 * H * r) * 2.0)
+    cq = torch.randn(T, 2 * (W // 4), device=dev).to(bf)
+    add("rmsnorm_rows (query latent)", _timed(lambda: rmsnorm_rows(cq[:, : W // 4], torch.ones(W // 4, device=dev), 1e-6)),
+        bytes_=T * (W // 4) * 2 * 2.0)
+    # ---- sublayer boundary: S fp32 streams | one fp32 stream
+    xs = torch.randn(S, T, W, device=dev)
+    y = torch.randn(T, W, device=dev).to(bf)
+    mix, oc, ic, w32 = torch.eye(S, device=dev), torch.ones(S, device=dev), torch.ones(S, device=dev) / S, torch.ones(W, device=dev)
+    add(f"hyper_mix ({S} fp32 streams)", _timed(lambda: hyper_mix(xs, y, mix, oc, ic, w32, 1e-6)), bytes_=T * W * (2 + 8.0 * S + 2))
+    resid = torch.randn(T, W, device=dev)
+    b32 = torch.zeros(W, device=dev)
+    add("zofesun dyt_residual (one fp32 stream)", _timed(lambda: dyt_residual(resid, y, (0.5, w32, b32), pre=(0.5, w32, b32))),
+        bytes_=T * W * (2 + 4 + 4 + 2.0))
+    # ---- retention scan (rotary, no activation) | decay scan (SiLU) ; per-head | whole-row gated norm
+    pr = torch.randn(T, 4 * H * D, device=dev).to(bf)
+    dec = torch.full((H,), 0.99, device=dev)
+    St = torch.zeros(B + 1, H, D, D, device=dev)
+    add("retention scan prefill", _timed(lambda: decay_attention(pr, 0, H * D, 2 * H * D, dec, St, meta, H, D, D, act=False,
+                                                                positions=pos, rope=tab, k_scale=D ** -0.5), 3, 1),
+        flops=4.0 * T * H * D * D, bytes_=T * 3 * H * D * 2.0, peak=VALU_F32)
+    add("zofesun decay_attn_scan prefill", _timed(lambda: decay_attention(pr, 0, H * D, 2 * H * D, dec, St, meta, H, D, D), 3, 1),
+        flops=4.0 * T * H * D * D, bytes_=T * 3 * H * D * 2.0, peak=VALU_F32)
+    prd = torch.randn(B, 4 * H * D, device=dev).to(bf)
+    posd = torch.full((B,), ctx - 1, **i32)
+    add("retention scan decode", _timed(lambda: decay_attention(prd, 0, H * D, 2 * H * D, dec, St, dmeta, H, D, D, act=False,
+                                                               positions=posd, rope=tab, k_scale=D ** -0.5)),
+        bytes_=2.0 * B * H * D * D * 4)
+    add("zofesun decay_attn_scan decode", _timed(lambda: decay_attention(prd, 0, H * D, 2 * H * D, dec, St, dmeta, H, D, D)),
+        bytes_=2.0 * B * H * D * D * 4)
+    o = torch.randn(T, H * D, device=dev)
+    out = torch.empty(T, H * D, device=dev, dtype=bf)
+    add("gated_rmsnorm per head, SiLU gate", _timed(lambda: gated_rmsnorm(o, None, pr, 3 * H * D, 1e-6, out, groups=H, gate="silu")),
+        bytes_=T * H * D * (4 + 2 + 2.0))
+    add("zofesun gated_rmsnorm whole row", _timed(lambda: gated_rmsnorm(o, w32[: H * D].contiguous(), pr, 3 * H * D, 1e-5, out)),
+        bytes_=T * H * D * (4 + 2 + 2.0))
+    return rows
+
+
+def run_namudra(args) -> dict:
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    sizes = {}
+    for name in SIZES:
+        makers = dict(zip(("namudra", "zofesun", "qwen2"), _namudra_models(name, dev)))
+        cell = {}
+        for batch, plen, glen in ((8, 2048, 64), (64, 1024, 64)):
+            key = f"B{batch}_P{plen}_G{glen}"
+            cell[key] = {k: _engine_numbers(mk, dev, batch, plen, glen) for k, mk in makers.items()}
+            print(json.dumps({"size": name, "shape": key, **cell[key]}), flush=True)
+        sizes[name] = cell
+    kernels = _namudra_kernel_table(dev)
+    for r in kernels:
+        print(json.dumps(r), flush=True)
+    return {"metric": "namudra_vs_zofesun_vs_qwen2_tokens_per_s", "unit": "tokens/s", "dtype": "bf16",
+            "data": "synthetic", "sizes": sizes, "kernels": kernels}
+
+
 def run(args) -> dict:
+    if getattr(args, "hybrid", None) == "namudra":
+        return run_namudra(args)
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
     sizes = {}

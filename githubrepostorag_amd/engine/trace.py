@@ -23,10 +23,11 @@ SLOTS = 4  # live requests a replay may hold at once
 
 
 def run_trace(model_dir: str, dtype: str, out_dir: str, max_tokens: int, device: str | None = None,
-              block_size: int = 16, lines=None, log=sys.stdout) -> int:
+              block_size: int = 16, lines=None, log=None) -> int:
     from ..models import load_decoder
     from .llm_engine import EngineConfig, LLMEngine
 
+    log = sys.stdout if log is None else log  # (looked up per call: the caller may have swapped the stream)
     dt = {"bfloat16": torch.bfloat16, "float32": torch.float32}[dtype]
     dev = device or ("cuda" if torch.cuda.is_available() else "cpu")
     if dt == torch.float32:  # true fp32 products: no reduced-precision matrix modes

@@ -259,7 +259,7 @@ def case_window_edges(device, tol, dtype=torch.float32, bs=16):
         for j in range(ctx):
             kc[perm[j // bs], 0, j % bs, j] = 1.0
             vc[perm[j // bs], 0, j % bs] = V[j].to(dtype)
-        for qlen in (9, 1):
+        for qlen in (33, 9, 1):  # (33 queries in bf16: the matrix-core kernel)
             want = torch.zeros(qlen, H, d, dtype=torch.float64)
             q = torch.zeros(qlen, H, d)
             for n, p in enumerate(range(ctx - qlen, ctx)):
