@@ -96,6 +96,35 @@ rmsnorm_rows_kernel(const T* __restrict__ x, int ld, const float* __restrict__ w
   for (int i = threadIdx.x; i < N; i += 256) stg(out + (size_t)blockIdx.x * N + i, ldg(xr + i) * r * w[i]);
 }
 
+// bf16 rows of N % 8 == 0 columns, 16-byte aligned: 16-byte loads and stores, 8 columns per thread and pass.
+__global__ void __launch_bounds__(256)
+rmsnorm_rows_vec_kernel(const bf16* __restrict__ x, int ld, const float* __restrict__ w, bf16* __restrict__ out, int N,
+                        float eps) {
+  __shared__ float red[16];
+  const bf16* xr = x + (size_t)blockIdx.x * ld;
+  const int n8 = N >> 3;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < n8; c += blockDim.x) {
+    float f[8];
+    unpack8(*reinterpret_cast<const bf16x8_t*>(xr + c * 8), f);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ss = fmaf(f[e], f[e], ss);
+  }
+  ss = block_sum(ss, red);
+  const float r = 1.f / sqrtf(ss / (float)N + eps);
+  for (int c = threadIdx.x; c < n8; c += blockDim.x) {
+    float f[8];
+    unpack8(*reinterpret_cast<const bf16x8_t*>(xr + c * 8), f);
+    const f32x4_t w0 = *reinterpret_cast<const f32x4_t*>(w + c * 8), w1 = *reinterpret_cast<const f32x4_t*>(w + c * 8 + 4);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      f[e] *= r * w0[e];
+      f[e + 4] *= r * w1[e];
+    }
+    *reinterpret_cast<bf16x8_t*>(out + (size_t)blockIdx.x * N + c * 8) = pack8(f);
+  }
+}
+
 // ------------------------------------------------------------------------------------------------ q / k norm + store
 // proj [T, ld]: q heads at column qoff (H x d), k heads at koff (G x d).  q_out [T, H, d] = q / rms(q) * qw;
 // k_cache [nblk, G, BS, d] <- k / rms(k) * kw; v_cache [nblk, G, BS, d] <- k as projected (the values are the keys).
@@ -555,6 +584,12 @@ GRAG_API hipError_t grag_hyper_mix(float* streams, int S, const void* y, const f
 GRAG_API hipError_t grag_rmsnorm_rows(const void* x, int ld, const float* w, void* out, int T_, int N, float eps,
                                       int dt, hipStream_t st) {
   if (T_ <= 0) return hipSuccess;
+  auto al16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+  if (dt == 0 && N % 8 == 0 && ld % 8 == 0 && al16(x) && al16(w) && al16(out)) {
+    hipLaunchKernelGGL(rmsnorm_rows_vec_kernel, dim3(T_), dim3(N <= 1024 ? 128 : 256), 0, st, (const bf16*)x, ld, w,
+                       (bf16*)out, N, eps);
+    return hipGetLastError();
+  }
   DT_DISPATCH(dt, hipLaunchKernelGGL(rmsnorm_rows_kernel<T>, dim3(T_), dim3(256), 0, st, (const T*)x, ld, w, (T*)out,
                                      N, eps);)
   return hipGetLastError();
@@ -641,6 +676,12 @@ GRAG_API hipError_t grag_sigmoid_window_prefill(const void* q, const void* k_cac
   return hipGetLastError();
 }
 
+extern "C" hipError_t grag_window_decode_mfma(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                              int out_ld, const int* block_tables, int bt_stride, const int* ctx_len,
+                                              const float* bias, int nseq, int H, int G, int d, int vd, int BS,
+                                              float scale, int window, int nblocks, const void* gate, int gate_ld,
+                                              hipStream_t st);
+
 GRAG_API hipError_t grag_sigmoid_window_decode(const void* q, const void* k_cache, const void* v_cache, void* out,
                                                int out_ld, const int* block_tables, int bt_stride, const int* ctx_len,
                                                const float* bias, int nseq, int H, int G, int d, int vd, int BS,
@@ -648,6 +689,11 @@ GRAG_API hipError_t grag_sigmoid_window_decode(const void* q, const void* k_cach
                                                int gate_ld, hipStream_t st) {
   if (nseq <= 0) return hipSuccess;
   if (vd > 64 * SW_VC || G < 1 || H % G || window < 1) return hipErrorInvalidValue;
+  if (dt == 0) {  // bf16: the heads of a kv head share its keys on the matrix cores (seqmix.hip), when the sizes fit
+    const hipError_t e = grag_window_decode_mfma(q, k_cache, v_cache, out, out_ld, block_tables, bt_stride, ctx_len,
+                                                 bias, nseq, H, G, d, vd, BS, scale, window, nblocks, gate, gate_ld, st);
+    if (e != hipErrorNotSupported) return e;
+  }
   const size_t bytes = ((size_t)d + 4 * 64 + 4 * (size_t)vd) * sizeof(float);
   DT_DISPATCH(dt, hipLaunchKernelGGL(sigmoid_window_decode_kernel<T>, dim3(H, nseq), dim3(256), bytes, st, (const T*)q,
                                      (const T*)k_cache, (const T*)v_cache, (T*)out, out_ld, block_tables, bt_stride,

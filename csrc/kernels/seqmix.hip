@@ -462,18 +462,25 @@ sink_attn_prefill_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict
 // its own running (max, sum, O) and the four waves merge through LDS at the end.  With nsplit > 1 every split
 // writes its unnormalised O and (max, sum) to part_o [nsplit, nseq, H, vd] / part_ml [nsplit, nseq, H, 2] and
 // sink_attn_combine_kernel merges them; the sink term enters once (split 0, wave 0).
-template <int NKM, int NVM>
+//
+// More than 16 heads per kv head (one shared kv head under many heads): grid.y = G * ceil(R / 16), every block takes
+// a group of up to 16 of them.  SIG = 1 turns the kernel into sliding-window attention with sigmoid weights:
+// `sinks` then holds the per-head bias, the keys are the last `window` ones (one split), a key's weight is
+// sigmoid(score * scale + bias) with no running maximum and no normaliser, the waves' sums are added, and the
+// output is multiplied by sigmoid(gate) when a gate row is given.
+template <int NKM, int NVM, int SIG>
 __global__ void __launch_bounds__(256, NKM <= 8 && NVM <= 8 ? 3 : 2)
 sink_attn_decode_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_cache,
                              const bf16* __restrict__ v_cache, bf16* __restrict__ out, int out_ld,
                              const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ ctx_len,
                              const float* __restrict__ sinks, int H, int G, int d, int vd, int BS, float scale,
                              float out_scale, int nblocks, int nsplit, int split_len, float* __restrict__ part_o,
-                             float* __restrict__ part_ml) {
+                             float* __restrict__ part_ml, int window, const bf16* __restrict__ gate, int gate_ld) {
   constexpr int KT = 64;
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
-  const int sp = blockIdx.x, g = blockIdx.y, seq = blockIdx.z, nseq = gridDim.z;
-  const int R = H / G;
+  const int R = H / G, ngrp = (R + 15) >> 4;
+  const int sp = blockIdx.x, g = blockIdx.y / ngrp, hg = (blockIdx.y - g * ngrp) * 16, seq = blockIdx.z,
+            nseq = gridDim.z;
   const int ctx = ctx_len[seq];
   const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
   const int ql = lane & 15, quad = lane >> 4;
@@ -481,8 +488,8 @@ sink_attn_decode_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict_
   const int kstride = d + 8, vstride = vd * 4 + 8;  // vstride: one 4-key group of V
   short* Ks = reinterpret_cast<short*>(smem_raw);
   short* Vs = Ks + KT * kstride;
-  const bool col_ok = ql < R;
-  const int head = g * R + (col_ok ? ql : 0);
+  const bool col_ok = hg + ql < R;
+  const int head = g * R + (col_ok ? hg + ql : 0);
   bf16x4_t qf[NKM];
 #pragma unroll
   for (int ks = 0; ks < NKM; ++ks) {
@@ -490,13 +497,14 @@ sink_attn_decode_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict_
     if (ks < nk && col_ok)
       qf[ks] = *reinterpret_cast<const bf16x4_t*>(q + ((size_t)seq * H + head) * d + ks * 16 + quad * 4);
   }
-  const bool has_sink = sp == 0 && wid == 0;
+  const bool has_sink = !SIG && sp == 0 && wid == 0;
   float m = has_sink ? sinks[head] : -INFINITY, l = has_sink ? 1.f : 0.f;
+  const float pb = SIG ? sinks[head] : 0.f;
   f32x4_t acc[NVM];
 #pragma unroll
   for (int v = 0; v < NVM; ++v) acc[v] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  const int kbeg = nsplit > 1 ? sp * split_len : 0;
-  const int kend = nsplit > 1 ? min(ctx, kbeg + split_len) : ctx;
+  const int kbeg = SIG ? max(0, ctx - window) : nsplit > 1 ? sp * split_len : 0;
+  const int kend = SIG ? ctx : nsplit > 1 ? min(ctx, kbeg + split_len) : ctx;
   const int* bt = block_tables + (size_t)seq * bt_stride;
   bf16x8_t kreg[NKM / 2], vreg[NVM / 2];
   RowCursor rc;
@@ -527,42 +535,56 @@ sink_attn_decode_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict_
         st = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, qf[ks], st, 0, 0, 0);
       }
     }
-    float tmax = -INFINITY;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const bool vis = col_ok && 16 * wid + 4 * quad + i < kn;
-      st[i] = vis ? st[i] * scale : -INFINITY;
-      tmax = fmaxf(tmax, st[i]);
-    }
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-    const float mn = fmaxf(m, tmax);
-    const float alpha = m == -INFINITY ? 0.f : expf(m - mn);
-    float psum = 0.f;
     bf16x4_t ph, pl;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const float p = st[i] == -INFINITY ? 0.f : expf(st[i] - mn);
-      psum += p;
-      const short hi = f2bits(p);
-      ph[i] = hi;
-      pl[i] = f2bits(p - bits2f(hi));
-    }
-    psum += __shfl_xor(psum, 16, 64);
-    psum += __shfl_xor(psum, 32, 64);
-    l = l * alpha + psum;
-    m = mn;
     float arow[4];  // rescale factors of the accumulator rows (heads 4*quad + i)
+    if (SIG) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) arow[i] = __shfl(alpha, 4 * quad + i, 64);
+      for (int i = 0; i < 4; ++i) {
+        const bool vis = col_ok && 16 * wid + 4 * quad + i < kn;
+        const float p = vis ? sigmoid_acc(fmaf(st[i], scale, pb)) : 0.f;
+        const short hi = f2bits(p);
+        ph[i] = hi;
+        pl[i] = f2bits(p - bits2f(hi));
+        arow[i] = 1.f;
+      }
+    } else {
+      float tmax = -INFINITY;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const bool vis = col_ok && 16 * wid + 4 * quad + i < kn;
+        st[i] = vis ? st[i] * scale : -INFINITY;
+        tmax = fmaxf(tmax, st[i]);
+      }
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+      const float mn = fmaxf(m, tmax);
+      const float alpha = m == -INFINITY ? 0.f : expf(m - mn);
+      float psum = 0.f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float p = st[i] == -INFINITY ? 0.f : expf(st[i] - mn);
+        psum += p;
+        const short hi = f2bits(p);
+        ph[i] = hi;
+        pl[i] = f2bits(p - bits2f(hi));
+      }
+      psum += __shfl_xor(psum, 16, 64);
+      psum += __shfl_xor(psum, 32, 64);
+      l = l * alpha + psum;
+      m = mn;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) arow[i] = __shfl(alpha, 4 * quad + i, 64);
+    }
     const short* vr = Vs + (4 * wid + quad) * vstride + ql * 4;
 #pragma unroll
     for (int v = 0; v < NVM; ++v) {
       if (v < nv) {
         // V[keys 16w + 4*quad + 0..3][value dim 16v + ql]
         const bf16x4_t b = *reinterpret_cast<const bf16x4_t*>(vr + 64 * v);
+        if (!SIG) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) acc[v][i] *= arow[i];
+          for (int i = 0; i < 4; ++i) acc[v][i] *= arow[i];
+        }
         acc[v] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(ph, b, acc[v], 0, 0, 0);
         acc[v] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(pl, b, acc[v], 0, 0, 0);
       }
@@ -591,7 +613,11 @@ sink_attn_decode_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict_
     f[w] = mw == -INFINITY ? 0.f : expf(mw - M);
     L += Lw[w * 16 + ql] * f[w];
   }
-  if (nsplit > 1 && wid == 0 && quad == 0 && col_ok) {
+  if (SIG) {  // plain sums: every wave's part counts as it is
+    f[0] = f[1] = f[2] = f[3] = 1.f;
+    L = 1.f;
+  }
+  if (!SIG && nsplit > 1 && wid == 0 && quad == 0 && col_ok) {
     float* ml = part_ml + (((size_t)sp * nseq + seq) * H + head) * 2;
     ml[0] = M;
     ml[1] = L;
@@ -603,17 +629,18 @@ sink_attn_decode_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict_
 #pragma unroll
     for (int w = 0; w < 4; ++w) fr[w] = __shfl(f[w], r, 64);
     const float Lr = __shfl(L, r, 64);
-    if (r >= R) continue;
-    const int hr = g * R + r;
+    if (hg + r >= R) continue;
+    const int hr = g * R + hg + r;
 #pragma unroll
     for (int v = 0; v < NVM; ++v) {
       if (v < nv && (v & 3) == wid) {
         float x = 0.f;
         for (int w = 0; w < 4; ++w) x = fmaf(Aw[((size_t)w * 16 + r) * vd + 16 * v + ql], fr[w], x);
-        if (nsplit > 1) {
+        if (!SIG && nsplit > 1) {
           part_o[(((size_t)sp * nseq + seq) * H + hr) * vd + 16 * v + ql] = x;
         } else {
-          out[(size_t)seq * out_ld + hr * vd + 16 * v + ql] = (bf16)(x * (out_scale / Lr));
+          const float gt = (SIG && gate) ? sigmoid_acc((float)gate[(size_t)seq * gate_ld + hr * vd + 16 * v + ql]) : 1.f;
+          out[(size_t)seq * out_ld + hr * vd + 16 * v + ql] = (bf16)(x * (out_scale / Lr) * gt);
         }
       }
     }
@@ -1012,6 +1039,38 @@ __global__ void gated_rmsnorm_kernel(const float* __restrict__ x, const float* _
   }
 }
 
+// the same with one wave per group (groups of at most a few hundred columns: heads): grid (T, ceil(groups / 4)), no
+// block-level barrier, the group's values stay in registers between the two passes (up to 8 per lane).
+template <typename T>
+__global__ void __launch_bounds__(256)
+gated_rmsnorm_wave_kernel(const float* __restrict__ x, const float* __restrict__ w, const T* __restrict__ proj, int ld,
+                          int goff, T* __restrict__ out, int out_ld, int N, int groups, float eps, float out_scale,
+                          int silu_gate) {
+  const int t = blockIdx.x, grp = blockIdx.y * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (grp >= groups) return;
+  const int c0 = grp * N;
+  const float* xr = x + (size_t)t * N * groups + c0;
+  float v[8];
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    const int i = lane + 64 * k;
+    v[k] = i < N ? xr[i] : 0.f;
+    ss = fmaf(v[k], v[k], ss);
+  }
+  ss = wave_sum(ss);
+  const float r = out_scale / sqrtf(ss / (float)N + eps);
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    const int i = lane + 64 * k;
+    if (i < N) {
+      const float g = ldf(proj + (size_t)t * ld + goff + c0 + i);
+      const float gt = silu_gate ? silu_acc(g) : sigmoid_acc(g);
+      stf(out + (size_t)t * out_ld + c0 + i, v[k] * r * (w ? w[c0 + i] : 1.f) * gt);
+    }
+  }
+}
+
 // ------------------------------------------------------------------------------------------------ minGRU
 // z = sigmoid(pz + bz), u = px + bx, c = u >= 0 ? u + 1/2 : sigmoid(u); S_t = (1 - z) S_(t-1) + z c;
 // out = S_t * silu(pg).  grid (ceil(W / 256), nseq): one thread per channel walks the launch's tokens in order.
@@ -1237,24 +1296,25 @@ GRAG_API hipError_t grag_sink_attn_decode(const void* q, const void* k_cache, co
                                           int split_len, float* part_o, float* part_ml, hipStream_t st) {
   if (nseq <= 0) return hipSuccess;
   if (vd > 64 * SA_VC || G <= 0 || H % G) return hipErrorInvalidValue;
-  if (dt == 0 && d % 16 == 0 && vd % 16 == 0 && d <= 256 && vd <= 256 && H / G <= 16 && out_ld % 4 == 0 &&
-      (reinterpret_cast<uintptr_t>(out) & 7) == 0 && (reinterpret_cast<uintptr_t>(q) & 7) == 0 && nseq <= 65535) {
+  if (dt == 0 && d % 16 == 0 && vd % 16 == 0 && d <= 256 && vd <= 256 && G * ((H / G + 15) / 16) <= 65535 &&
+      out_ld % 4 == 0 && (reinterpret_cast<uintptr_t>(out) & 7) == 0 && (reinterpret_cast<uintptr_t>(q) & 7) == 0 &&
+      nseq <= 65535) {
     if (nsplit < 1 || part_o == nullptr || part_ml == nullptr || split_len % 64) nsplit = 1;
     const size_t kvb = ((size_t)64 * (d + 8) + (size_t)16 * (vd * 4 + 8)) * sizeof(short);
     const size_t mgb = (128 + (size_t)4 * vd * 16) * sizeof(float);
     const size_t mb = kvb > mgb ? kvb : mgb;
-    const dim3 mgrid(nsplit, G, nseq);
+    const dim3 mgrid(nsplit, G * ((H / G + 15) / 16), nseq);
 #define SD_MFMA(NK, NV)                                                                                              \
   {                                                                                                                  \
     if (mb > 48 * 1024) {                                                                                            \
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&sink_attn_decode_mfma_kernel<NK, NV>),       \
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&sink_attn_decode_mfma_kernel<NK, NV, 0>),    \
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)mb);                       \
       if (e != hipSuccess) return e;                                                                                 \
     }                                                                                                                \
-    hipLaunchKernelGGL((sink_attn_decode_mfma_kernel<NK, NV>), mgrid, dim3(256), mb, st, (const bf16*)q,             \
+    hipLaunchKernelGGL((sink_attn_decode_mfma_kernel<NK, NV, 0>), mgrid, dim3(256), mb, st, (const bf16*)q,          \
                        (const bf16*)k_cache, (const bf16*)v_cache, (bf16*)out, out_ld, block_tables, bt_stride,      \
                        ctx_len, sinks, H, G, d, vd, BS, scale, out_scale, nblocks, nsplit, split_len, part_o,        \
-                       part_ml);                                                                                     \
+                       part_ml, 0, (const bf16*)nullptr, 0);                                                         \
   }
     const int nk = d / 16, nv = vd / 16;
     if (nk <= 4 && nv <= 4) SD_MFMA(4, 4)
@@ -1278,6 +1338,39 @@ GRAG_API hipError_t grag_sink_attn_decode(const void* q, const void* k_cache, co
   DT_DISPATCH(dt, hipLaunchKernelGGL(sink_attn_decode_kernel<T>, dim3(H, nseq), dim3(256), bytes, st, (const T*)q,
                                      (const T*)k_cache, (const T*)v_cache, (T*)out, out_ld, block_tables, bt_stride,
                                      ctx_len, sinks, H, G, d, vd, BS, scale, out_scale, nblocks);)
+  return hipGetLastError();
+}
+
+// Sliding-window decode with sigmoid weights on the matrix cores (bf16; the SIG form of the kernel above): returns
+// hipErrorNotSupported when the shapes do not fit it, and the caller takes its vector kernel.
+GRAG_API hipError_t grag_window_decode_mfma(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                            int out_ld, const int* block_tables, int bt_stride, const int* ctx_len,
+                                            const float* bias, int nseq, int H, int G, int d, int vd, int BS,
+                                            float scale, int window, int nblocks, const void* gate, int gate_ld,
+                                            hipStream_t st) {
+  if (nseq <= 0) return hipSuccess;
+  if (G <= 0 || H % G || d % 16 || vd % 16 || d > 128 || vd > 128 || G * ((H / G + 15) / 16) > 65535 || nseq > 65535 ||
+      (reinterpret_cast<uintptr_t>(q) & 7))
+    return hipErrorNotSupported;
+  const size_t kvb = ((size_t)64 * (d + 8) + (size_t)16 * (vd * 4 + 8)) * sizeof(short);
+  const size_t mgb = (128 + (size_t)4 * vd * 16) * sizeof(float);
+  const size_t mb = kvb > mgb ? kvb : mgb;
+  const dim3 mgrid(1, G * ((H / G + 15) / 16), nseq);
+#define SW_MFMA(NK, NV)                                                                                              \
+  {                                                                                                                  \
+    if (mb > 48 * 1024) {                                                                                            \
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&sink_attn_decode_mfma_kernel<NK, NV, 1>),    \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)mb);                       \
+      if (e != hipSuccess) return e;                                                                                 \
+    }                                                                                                                \
+    hipLaunchKernelGGL((sink_attn_decode_mfma_kernel<NK, NV, 1>), mgrid, dim3(256), mb, st, (const bf16*)q,          \
+                       (const bf16*)k_cache, (const bf16*)v_cache, (bf16*)out, out_ld, block_tables, bt_stride,      \
+                       ctx_len, bias, H, G, d, vd, BS, scale, 1.f, nblocks, 1, 0, (float*)nullptr, (float*)nullptr,  \
+                       window, (const bf16*)gate, gate_ld);                                                          \
+  }
+  if (d <= 64 && vd <= 64) SW_MFMA(4, 4)
+  else SW_MFMA(8, 8)
+#undef SW_MFMA
   return hipGetLastError();
 }
 
@@ -1345,6 +1438,12 @@ GRAG_API hipError_t grag_gated_rmsnorm(const float* x, const float* w, const voi
                                        int silu_gate, hipStream_t st) {
   if (T_ <= 0) return hipSuccess;
   if (groups < 1 || groups > 65535 || N % groups) return hipErrorInvalidValue;
+  if (groups > 1 && N / groups <= 512) {
+    DT_DISPATCH(dt, hipLaunchKernelGGL(gated_rmsnorm_wave_kernel<T>, dim3(T_, (groups + 3) / 4), dim3(256), 0, st, x, w,
+                                       (const T*)proj, ld, goff, (T*)out, out_ld, N / groups, groups, eps, out_scale,
+                                       silu_gate);)
+    return hipGetLastError();
+  }
   const int threads = N / groups <= 64 ? 64 : N / groups <= 128 ? 128 : 256;
   DT_DISPATCH(dt, hipLaunchKernelGGL(gated_rmsnorm_kernel<T>, dim3(T_, groups), dim3(threads), 0, st, x, w,
                                      (const T*)proj, ld, goff, (T*)out, out_ld, N / groups, eps, out_scale, silu_gate);)

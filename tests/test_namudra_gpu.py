@@ -125,6 +125,21 @@ def test_matrix_core_shapes_bf16():
     assert C.rel_err(C.feed_in_portions(eng, "c", toks, [64, 70, 50] + [1] * 16), want) < BF16
 
 
+def test_more_than_sixteen_heads_per_kv_head_bf16():
+    """Decode kernels that pack the heads of one kv head into 16 matrix-core columns take them in groups: 18 heads
+    on one kv head (windowed attention), 20 heads on the latent cache."""
+    cfg = O.make_config(width=64, kinds=("attention", "latent_attention"), loop=(0, 0, 1), no_mlp=(0,),
+                        att=dict(heads=18, kv_heads=1, dim=16, vdim=16, scale=0.3, mask={"size": 50}),
+                        lat=dict(heads=20, dim=16, rot_dim=16, vdim=16, kv_rank=32, q_rank=32, scale=0.25))
+    sd = O.make_weights(cfg, seed=53)
+    toks = C.tokens(cfg, 120, 9)
+    want = O.forward(cfg, sd, toks)
+    _, eng = C.build(cfg, sd, "cuda", torch.bfloat16)
+    assert C.rel_err(C.feed_in_portions(eng, "c", toks, [90] + [1] * 30), want) < BF16
+    _, eng = C.build(cfg, sd, "cuda", torch.float32)
+    assert C.rel_err(C.feed_in_portions(eng, "d", toks, [90] + [1] * 30), want) < F32
+
+
 @pytest.mark.parametrize("graphs,mixed,window,max_batched", [(False, False, 1, 4096), (True, False, 1, 4096),
                                                              (True, False, 4, 4096), (False, True, 1, 8)])
 def test_greedy_generation(graphs, mixed, window, max_batched):
