@@ -77,6 +77,82 @@ hyper_mix_kernel(float* __restrict__ streams, size_t sstride, int S, const T* __
   for (int i = threadIdx.x; i < H; i += 256) stg(out + row + i, us[i] * r * w[i]);
 }
 
+// H % 4 == 0 and 16-byte aligned rows: four consecutive columns per thread and step (16-byte loads and stores of the
+// streams, 8- or 16-byte loads of y), otherwise the same pass.
+template <typename T> __device__ __forceinline__ f32x4_t ld4(const T* p);
+template <> __device__ __forceinline__ f32x4_t ld4<float>(const float* p) { return *reinterpret_cast<const f32x4_t*>(p); }
+template <> __device__ __forceinline__ f32x4_t ld4<bf16>(const bf16* p) {
+  const bf16x4_t v = *reinterpret_cast<const bf16x4_t*>(p);
+  return f32x4_t{bits2f(v[0]), bits2f(v[1]), bits2f(v[2]), bits2f(v[3])};
+}
+template <typename T> __device__ __forceinline__ void st4(T* p, const f32x4_t& v);
+template <> __device__ __forceinline__ void st4<float>(float* p, const f32x4_t& v) { *reinterpret_cast<f32x4_t*>(p) = v; }
+template <> __device__ __forceinline__ void st4<bf16>(bf16* p, const f32x4_t& v) {
+  *reinterpret_cast<bf16x4_t*>(p) = bf16x4_t{f2bits(v[0]), f2bits(v[1]), f2bits(v[2]), f2bits(v[3])};
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+hyper_mix_vec_kernel(float* __restrict__ streams, size_t sstride, int S, const T* __restrict__ y,
+                     const float* __restrict__ mix, const float* __restrict__ outc, const float* __restrict__ inc,
+                     const float* __restrict__ w, float eps, T* __restrict__ out, float* __restrict__ out_sum, int H) {
+  extern __shared__ __attribute__((aligned(16))) float us[];
+  __shared__ float red[16];
+  const size_t row = (size_t)blockIdx.x * H;
+  float ss = 0.f;
+  for (int i = threadIdx.x * 4; i < H; i += 1024) {
+    f32x4_t x[HC_MAX];
+#pragma unroll
+    for (int s = 0; s < HC_MAX; ++s)
+      x[s] = s < S ? *reinterpret_cast<const f32x4_t*>(streams + s * sstride + row + i) : f32x4_t{0.f, 0.f, 0.f, 0.f};
+    if (y != nullptr) {
+      const f32x4_t yi = ld4(y + row + i);
+      f32x4_t n[HC_MAX];
+#pragma unroll
+      for (int t = 0; t < HC_MAX; ++t) {
+        f32x4_t a = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        if (t < S) {
+#pragma unroll
+          for (int s = 0; s < HC_MAX; ++s)
+            if (s < S) {
+              const float m = mix[s * S + t];
+#pragma unroll
+              for (int e = 0; e < 4; ++e) a[e] = fmaf(m, x[s][e], a[e]);
+            }
+          const float oc = outc[t];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) a[e] = fmaf(oc, yi[e], a[e]);
+          *reinterpret_cast<f32x4_t*>(streams + t * sstride + row + i) = a;
+        }
+        n[t] = a;
+      }
+#pragma unroll
+      for (int t = 0; t < HC_MAX; ++t) x[t] = n[t];
+    }
+    if (inc != nullptr) {
+      f32x4_t u = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < HC_MAX; ++s)
+        if (s < S) {
+          const float c = inc[s];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) u[e] = fmaf(c, x[s][e], u[e]);
+        }
+      *reinterpret_cast<f32x4_t*>(us + i) = u;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) ss = fmaf(u[e], u[e], ss);
+      if (out_sum != nullptr) *reinterpret_cast<f32x4_t*>(out_sum + row + i) = u;
+    }
+  }
+  if (inc == nullptr || out == nullptr) return;
+  ss = block_sum(ss, red);
+  const float r = 1.f / sqrtf(ss / (float)H + eps);
+  for (int i = threadIdx.x * 4; i < H; i += 1024) {
+    const f32x4_t u = *reinterpret_cast<const f32x4_t*>(us + i), wv = *reinterpret_cast<const f32x4_t*>(w + i);
+    st4(out + row + i, f32x4_t{u[0] * r * wv[0], u[1] * r * wv[1], u[2] * r * wv[2], u[3] * r * wv[3]});
+  }
+}
+
 // ------------------------------------------------------------------------------------------------ RMS norm of column slices
 // out [T, N] = x / sqrt(mean(x^2) + eps) * w for rows x of stride ld (a column slice of a fused projection).
 // grid (T), 256 threads.
@@ -569,6 +645,12 @@ GRAG_API hipError_t grag_hyper_mix(float* streams, int S, const void* y, const f
   if (y != nullptr && (mix == nullptr || outc == nullptr)) return hipErrorInvalidValue;
   if (out != nullptr && (inc == nullptr || w == nullptr)) return hipErrorInvalidValue;
   const size_t bytes = (size_t)H * sizeof(float);
+  auto al16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+  if (H % 4 == 0 && bytes <= 48 * 1024 && al16(streams) && al16(y) && al16(w) && al16(out) && al16(out_sum)) {
+    DT_DISPATCH(dt, hipLaunchKernelGGL(hyper_mix_vec_kernel<T>, dim3(T_), dim3(256), bytes, st, streams,
+                                       (size_t)T_ * H, S, (const T*)y, mix, outc, inc, w, eps, (T*)out, out_sum, H);)
+    return hipGetLastError();
+  }
   DT_DISPATCH(dt, {
     if (bytes > 48 * 1024) {
       hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&hyper_mix_kernel<T>),

@@ -158,7 +158,7 @@ __global__ void rope_vnorm_store_kernel(const T* __restrict__ proj, int ld, int 
 // softmax over the visible keys plus one key-less, value-less term exp(sink_h) in the denominator: the running
 // (max, sum) starts at (sink_h, 1) instead of (-inf, 0).
 constexpr int SA_NQ = 4;   // queries per wave (prefill)
-constexpr int SA_VC = 4;   // 64-wide value-dim chunks per lane: vd <= 256
+constexpr int SA_VC = 8;   // 64-wide value-dim chunks per lane: vd <= 512 (a latent cache's value row can be that wide)
 
 // prefill: grid (q tiles of 4 waves x SA_NQ queries, H, nseq), 256 threads.  A tile of KT keys (K [KT][d+1] and
 // V [KT][vd], fp32) is staged in LDS per step; lane = key for the scores, lane = value dim for the output.

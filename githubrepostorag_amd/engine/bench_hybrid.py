@@ -243,10 +243,11 @@ def _namudra_kernel_table(dev, H=28, G=4, D=128, W=3584, T=2048, B=64, ctx=2048,
                                                                     H, G, D, D, D, 1e-5)), bytes_=T * (H + 2 * G) * D * 2 * 2.0)
     ckv = torch.randn(T, R + r, device=dev).to(bf)
     tabr = rope_table(T, r, 1e4, dev)
-    add("latent_store", _timed(lambda: latent_store(ckv, torch.ones(R, device=dev), pos, tabr, meta.slot_mapping, ql, kl, vl, 1e-6)),
+    wR, wq4 = torch.ones(R, device=dev), torch.ones(W // 4, device=dev)
+    add("latent_store", _timed(lambda: latent_store(ckv, wR, pos, tabr, meta.slot_mapping, ql, kl, vl, 1e-6)),
         bytes_=T * ((R + r) * 2 + R + 2 * H * r) * 2.0)
     cq = torch.randn(T, 2 * (W // 4), device=dev).to(bf)
-    add("rmsnorm_rows (query latent)", _timed(lambda: rmsnorm_rows(cq[:, : W // 4], torch.ones(W // 4, device=dev), 1e-6)),
+    add("rmsnorm_rows (query latent)", _timed(lambda: rmsnorm_rows(cq[:, : W // 4], wq4, 1e-6)),
         bytes_=T * (W // 4) * 2 * 2.0)
     # ---- sublayer boundary: S fp32 streams | one fp32 stream
     xs = torch.randn(S, T, W, device=dev)

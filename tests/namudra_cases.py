@@ -190,6 +190,9 @@ def case_other_sizes(device, tol, dtype=torch.float32):
               lat=dict(heads=5, dim=4, rot_dim=12, vdim=4, kv_rank=8, q_rank=24, scale=0.7)), True),
         # three streams, a loop that runs once, a window of two
         (dict(streams=3, loop=(1, 2, 1), att=dict(mask={"size": 2})), True),
+        # a latent wider than the matrix-core kernels' rows (value row above 256)
+        (dict(kinds=("latent_attention",), loop=(0, 0, 1), no_mlp=(),
+              lat=dict(heads=2, dim=8, rot_dim=8, vdim=8, kv_rank=320, q_rank=16, scale=0.2)), True),
     ]
     for i, (kw, hc) in enumerate(variants):
         cfg = O.make_config(**kw)
