@@ -125,6 +125,22 @@ def test_matrix_core_shapes_bf16():
     assert C.rel_err(C.feed_in_portions(eng, "c", toks, [64, 70, 50] + [1] * 16), want) < BF16
 
 
+def test_serving_head_sizes_bf16():
+    """The head sizes of the bench presets (128-wide heads, a latent of 192 + 64 rotated: key rows of 256) at a small
+    width: the widest instantiations of the matrix-core kernels, prompts and decoded tokens."""
+    cfg = O.make_config(width=128, vocab=128, kinds=("retention", "attention", "latent_attention"), loop=(0, 0, 1),
+                        no_mlp=(0, 1, 2), ret=dict(heads=2, dim=128, vdim=128, decay=[0.98, 0.999], rot={"dims": 128, "base": 1e4}),
+                        att=dict(heads=4, kv_heads=2, dim=128, vdim=128, scale=0.09, mask={"size": 80}),
+                        lat=dict(heads=4, dim=128, rot_dim=64, vdim=128, kv_rank=192, q_rank=96, scale=0.07))
+    sd = O.make_weights(cfg, seed=57)
+    toks = C.tokens(cfg, 150, 11)
+    want = O.forward(cfg, sd, toks)
+    _, eng = C.build(cfg, sd, "cuda", torch.bfloat16)
+    assert C.rel_err(C.feed_in_portions(eng, "c", toks, [70, 64] + [1] * 16), want) < BF16
+    _, eng = C.build(cfg, sd, "cuda", torch.float32)
+    assert C.rel_err(C.feed_in_portions(eng, "d", toks, [70, 64] + [1] * 16), want) < F32
+
+
 def test_more_than_sixteen_heads_per_kv_head_bf16():
     """Decode kernels that pack the heads of one kv head into 16 matrix-core columns take them in groups: 18 heads
     on one kv head (windowed attention), 20 heads on the latent cache."""
