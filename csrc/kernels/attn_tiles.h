@@ -37,9 +37,10 @@ __device__ __forceinline__ int tile_block(const RowCursor& rc, const int* __rest
 }
 template <int NL>
 __device__ __forceinline__ void tile_load(bf16x8_t (&reg)[NL], const bf16* __restrict__ cache, int blk, int off,
-                                          int rowlen, int G, int g, int BS) {
+                                          int rowlen, int G, int g, int BS, int stride = -1) {
+  // (stride: elements from one cached row to the next, when the rows read are the head of wider ones)
   const int r8 = rowlen >> 3;
-  const bf16* row = cache + (((size_t)(blk < 0 ? 0 : blk) * G + g) * BS + off) * rowlen;
+  const bf16* row = cache + (((size_t)(blk < 0 ? 0 : blk) * G + g) * BS + off) * (stride < 0 ? rowlen : stride);
 #pragma unroll
   for (int u = 0; u < NL; ++u) {
     const int c = (threadIdx.x & 3) + 4 * u;

@@ -2,8 +2,8 @@
 //   * hyper-connection boundary: S fp32 residual streams mixed by an S x S matrix, the sublayer's output added
 //     with one coefficient per stream, the next sublayer's input read out as a weighted sum and RMS-normed,
 //   * query / key RMS norm + paged store for attention whose values are the un-normed keys,
-//   * latent store: RMS-normed latent | rotated shared key part into a one-head paged cache, rotary on the rotated
-//     tail of every (absorbed) query head,
+//   * latent store: RMS-normed latent | rotated shared key part into the rows of a one-head paged cache, rotary on the
+//     rotated tail of every (absorbed) query head,
 //   * sliding-window attention with sigmoid weights (no softmax, no normaliser), prefill and decode.
 // Activations are bf16 or fp32 (dt: 0 = bf16, 1 = fp32; the caches hold the same type); streams, norms, scores and
 // attention weights are fp32 in both.
@@ -242,16 +242,16 @@ qk_norm_store_kernel(const T* __restrict__ proj, int ld, int qoff, int koff, con
 
 // ------------------------------------------------------------------------------------------------ latent store
 // ckv [T, ld_c]: R latent columns, then r columns of the shared rotated key part.  k_cache [nblk, 1, BS, R + r] <-
-// latent / rms(latent) * cw | rotated part; v_cache [nblk, 1, BS, R] <- the normed latent again (the values of the
-// absorbed form).  q [T, H, R + r] (in place): the last r columns of every head are rotated.  Rotation: dim i paired
-// with i + r/2, table row p = cos[0:r/2] | sin[0:r/2] (fp32).
+// latent / rms(latent) * cw | rotated part (the values of the absorbed form are the first R columns of the same
+// rows).  q [T, H, R + r] (in place): the last r columns of every head are rotated.  Rotation: dim i paired with
+// i + r/2, table row p = cos[0:r/2] | sin[0:r/2] (fp32).
 // grid (T, ceil((1 + H) / 4)), 256 threads: wave 0 of a token owns the cache row, waves 1 .. H a query head each.
 template <typename T>
 __global__ void __launch_bounds__(256)
 latent_store_kernel(const T* __restrict__ ckv, int ld_c, const float* __restrict__ cw,
                     const int* __restrict__ positions, const float* __restrict__ table, int table_rows,
-                    const int* __restrict__ slot_mapping, T* __restrict__ q, T* __restrict__ k_cache,
-                    T* __restrict__ v_cache, int H, int R, int r, int BS, long nslots, float eps) {
+                    const int* __restrict__ slot_mapping, T* __restrict__ q, T* __restrict__ k_cache, int H, int R,
+                    int r, int BS, long nslots, float eps) {
   const int t = blockIdx.x, lane = threadIdx.x & 63;
   const int u = blockIdx.y * 4 + (threadIdx.x >> 6);
   if (u > H) return;
@@ -281,12 +281,7 @@ latent_store_kernel(const T* __restrict__ ckv, int ld_c, const float* __restrict
   ss = wave_sum(ss);
   const float rn = 1.f / sqrtf(ss / (float)R + eps);
   T* kd = k_cache + (size_t)slot * (R + r);
-  T* vd = v_cache + (size_t)slot * R;
-  for (int i = lane; i < R; i += 64) {
-    const float v = ldg(src + i) * rn * cw[i];
-    stg(kd + i, v);
-    stg(vd + i, v);
-  }
+  for (int i = lane; i < R; i += 64) stg(kd + i, ldg(src + i) * rn * cw[i]);
   for (int i = lane; i < half; i += 64) {
     const float a = ldg(src + R + i), b = ldg(src + R + i + half);
     const float c = cs[i], s = cs[half + i];
@@ -690,13 +685,13 @@ GRAG_API hipError_t grag_qk_norm_store(const void* proj, int ld, int qoff, int k
 
 GRAG_API hipError_t grag_latent_store(const void* ckv, int ld_c, const float* cw, const int* positions,
                                       const float* table, int table_rows, const int* slot_mapping, void* q,
-                                      void* k_cache, void* v_cache, int T_, int H, int R, int r, int BS, long nslots,
-                                      float eps, int dt, hipStream_t st) {
+                                      void* k_cache, int T_, int H, int R, int r, int BS, long nslots, float eps,
+                                      int dt, hipStream_t st) {
   if (T_ <= 0) return hipSuccess;
   if (H + 1 > 4 * 65535 || (r & 1)) return hipErrorInvalidValue;
   DT_DISPATCH(dt, hipLaunchKernelGGL(latent_store_kernel<T>, dim3(T_, (H + 4) / 4), dim3(256), 0, st, (const T*)ckv,
                                      ld_c, cw, positions, table, table_rows, slot_mapping, (T*)q, (T*)k_cache,
-                                     (T*)v_cache, H, R, r, BS, nslots, eps);)
+                                     H, R, r, BS, nslots, eps);)
   return hipGetLastError();
 }
 

@@ -168,7 +168,7 @@ sink_attn_prefill_kernel(const T* __restrict__ q, const T* __restrict__ k_cache,
                          T* __restrict__ out, int out_ld, const int* __restrict__ block_tables, int bt_stride,
                          const int* __restrict__ q_start, const int* __restrict__ ctx_len,
                          const float* __restrict__ sinks, int H, int G, int d, int vd, int BS, float scale,
-                         float out_scale, int KT, int nblocks) {
+                         float out_scale, int KT, int nblocks, int v_ld) {
   extern __shared__ float smem[];
   const int QT = 4 * SA_NQ;
   const int seq = blockIdx.z, h = blockIdx.y, g = h / (H / G);
@@ -216,7 +216,7 @@ sink_attn_prefill_kernel(const T* __restrict__ q, const T* __restrict__ k_cache,
       const int key = k0 + kk;
       const int blk = bt[key / BS];
       float v = 0.f;
-      if (blk >= 0 && blk < nblocks) v = ldf(v_cache + (((size_t)blk * G + g) * BS + key % BS) * vd + i);
+      if (blk >= 0 && blk < nblocks) v = ldf(v_cache + (((size_t)blk * G + g) * BS + key % BS) * v_ld + i);
       Vs[kk * vd + i] = v;
     }
     __syncthreads();
@@ -292,7 +292,7 @@ sink_attn_prefill_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict
                               const bf16* __restrict__ v_cache, bf16* __restrict__ out, int out_ld,
                               const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ q_start,
                               const int* __restrict__ ctx_len, const float* __restrict__ sinks, int H, int G, int d,
-                              int vd, int BS, float scale, float out_scale, int nblocks) {
+                              int vd, int BS, float scale, float out_scale, int nblocks, int v_ld) {
   constexpr int KT = 64;
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
   const int seq = blockIdx.z, h = blockIdx.y, g = h / (H / G);
@@ -338,7 +338,7 @@ sink_attn_prefill_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict
   {
     const int blk = tile_block(rc, bt, threadIdx.x >> 2, nkeys, nblocks, ERR_BLOCK_PREFILL);
     tile_load(kreg, k_cache, blk, rc.off, d, G, g, BS);
-    tile_load(vreg, v_cache, blk, rc.off, vd, G, g, BS);
+    tile_load(vreg, v_cache, blk, rc.off, vd, G, g, BS, v_ld);
   }
   for (int k0 = 0; k0 < nkeys; k0 += KT) {
     __syncthreads();
@@ -349,7 +349,7 @@ sink_attn_prefill_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict
       rc.advance(BS);
       const int blk = tile_block(rc, bt, k0 + KT + (threadIdx.x >> 2), nkeys, nblocks, ERR_BLOCK_PREFILL);
       tile_load(kreg, k_cache, blk, rc.off, d, G, g, BS);
-      tile_load(vreg, v_cache, blk, rc.off, vd, G, g, BS);
+      tile_load(vreg, v_cache, blk, rc.off, vd, G, g, BS, v_ld);
     }
     if (k0 > wave_qmax) continue;  // every key of the tile lies after this wave's queries
     f32x4_t st[4];
@@ -475,7 +475,8 @@ sink_attn_decode_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict_
                              const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ ctx_len,
                              const float* __restrict__ sinks, int H, int G, int d, int vd, int BS, float scale,
                              float out_scale, int nblocks, int nsplit, int split_len, float* __restrict__ part_o,
-                             float* __restrict__ part_ml, int window, const bf16* __restrict__ gate, int gate_ld) {
+                             float* __restrict__ part_ml, int window, const bf16* __restrict__ gate, int gate_ld,
+                             int v_ld) {
   constexpr int KT = 64;
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
   const int R = H / G, ngrp = (R + 15) >> 4;
@@ -512,7 +513,7 @@ sink_attn_decode_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict_
   if (kbeg < kend) {
     const int blk = tile_block(rc, bt, kbeg + (threadIdx.x >> 2), kend, nblocks, ERR_BLOCK_DECODE);
     tile_load(kreg, k_cache, blk, rc.off, d, G, g, BS);
-    tile_load(vreg, v_cache, blk, rc.off, vd, G, g, BS);
+    tile_load(vreg, v_cache, blk, rc.off, vd, G, g, BS, v_ld);
   }
   for (int k0 = kbeg; k0 < kend; k0 += KT) {
     __syncthreads();
@@ -523,7 +524,7 @@ sink_attn_decode_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict_
       rc.advance(BS);
       const int blk = tile_block(rc, bt, k0 + KT + (threadIdx.x >> 2), kend, nblocks, ERR_BLOCK_DECODE);
       tile_load(kreg, k_cache, blk, rc.off, d, G, g, BS);
-      tile_load(vreg, v_cache, blk, rc.off, vd, G, g, BS);
+      tile_load(vreg, v_cache, blk, rc.off, vd, G, g, BS, v_ld);
     }
     const int kn = min(KT, kend - k0);
     if (16 * wid >= kn) continue;  // this wave's 16 keys lie past the split's end
@@ -677,7 +678,7 @@ sink_attn_decode_vec_kernel(const bf16* __restrict__ q, const bf16* __restrict__
                             const bf16* __restrict__ v_cache, bf16* __restrict__ out, int out_ld,
                             const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ ctx_len,
                             const float* __restrict__ sinks, int H, int G, int d, int vd, int BS, float scale,
-                            float out_scale, int nblocks) {
+                            float out_scale, int nblocks, int v_ld) {
   extern __shared__ float smem[];
   const int seq = blockIdx.y, h = blockIdx.x, g = h / (H / G);
   const int ctx = ctx_len[seq];
@@ -731,7 +732,7 @@ sink_attn_decode_vec_kernel(const bf16* __restrict__ q, const bf16* __restrict__
           const int key2 = t * 64 + kk;
           int b2 = bt[key2 / BS];
           if (b2 < 0 || b2 >= nblocks) b2 = 0;
-          const uint32_t w = *reinterpret_cast<const uint32_t*>(v_cache + (((size_t)b2 * G + g) * BS + key2 % BS) * vd + j);
+          const uint32_t w = *reinterpret_cast<const uint32_t*>(v_cache + (((size_t)b2 * G + g) * BS + key2 % BS) * v_ld + j);
           const float pk = pw[kk];
           a0 = fmaf(pk, __uint_as_float(w << 16), a0);
           a1 = fmaf(pk, __uint_as_float(w & 0xffff0000u), a1);
@@ -779,7 +780,7 @@ __global__ void __launch_bounds__(256)
 sink_attn_decode_kernel(const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
                         T* __restrict__ out, int out_ld, const int* __restrict__ block_tables, int bt_stride,
                         const int* __restrict__ ctx_len, const float* __restrict__ sinks, int H, int G, int d, int vd,
-                        int BS, float scale, float out_scale, int nblocks) {
+                        int BS, float scale, float out_scale, int nblocks, int v_ld) {
   extern __shared__ float smem[];
   const int seq = blockIdx.y, h = blockIdx.x, g = h / (H / G);
   const int ctx = ctx_len[seq];
@@ -828,7 +829,7 @@ sink_attn_decode_kernel(const T* __restrict__ q, const T* __restrict__ k_cache, 
           const int key2 = t * 64 + kk;
           int b2 = bt[key2 / BS];
           if (b2 < 0 || b2 >= nblocks) b2 = 0;
-          a = fmaf(pw[kk], ldf(v_cache + (((size_t)b2 * G + g) * BS + key2 % BS) * vd + j), a);
+          a = fmaf(pw[kk], ldf(v_cache + (((size_t)b2 * G + g) * BS + key2 % BS) * v_ld + j), a);
         }
       }
       acc[c] = a;
@@ -1243,10 +1244,11 @@ GRAG_API hipError_t grag_sink_attn_prefill(const void* q, const void* k_cache, c
                                            int out_ld, const int* block_tables, int bt_stride, const int* q_start,
                                            const int* ctx_len, const float* sinks, int nseq, int max_q_len, int H,
                                            int G, int d, int vd, int BS, float scale, float out_scale, int nblocks,
-                                           int dt, hipStream_t st) {
+                                           int dt, int v_ld, hipStream_t st) {
+  // v_ld: elements from one cached value row to the next (vd, or more when the value rows are the head of wider rows)
   if (nseq <= 0 || max_q_len <= 0) return hipSuccess;
-  if (vd > 64 * SA_VC || G <= 0 || H % G) return hipErrorInvalidValue;
-  if (dt == 0 && max_q_len >= 16 && d % 16 == 0 && vd % 16 == 0 && d <= 256 && vd <= 256 && out_ld % 4 == 0 &&
+  if (vd > 64 * SA_VC || G <= 0 || H % G || v_ld < vd) return hipErrorInvalidValue;
+  if (dt == 0 && v_ld % 8 == 0 && (reinterpret_cast<uintptr_t>(v_cache) & 15) == 0 && max_q_len >= 16 && d % 16 == 0 && vd % 16 == 0 && d <= 256 && vd <= 256 && out_ld % 4 == 0 &&
       (reinterpret_cast<uintptr_t>(out) & 7) == 0 && (reinterpret_cast<uintptr_t>(q) & 7) == 0) {
     const size_t mb = ((size_t)64 * (d + 8) + (size_t)16 * (vd * 4 + 8)) * sizeof(short);
     const dim3 mgrid((max_q_len + 63) / 64, H, nseq);
@@ -1259,7 +1261,7 @@ GRAG_API hipError_t grag_sink_attn_prefill(const void* q, const void* k_cache, c
     }                                                                                                                \
     hipLaunchKernelGGL((sink_attn_prefill_mfma_kernel<NK, NV>), mgrid, dim3(256), mb, st, (const bf16*)q,            \
                        (const bf16*)k_cache, (const bf16*)v_cache, (bf16*)out, out_ld, block_tables, bt_stride,      \
-                       q_start, ctx_len, sinks, H, G, d, vd, BS, scale, out_scale, nblocks);                         \
+                       q_start, ctx_len, sinks, H, G, d, vd, BS, scale, out_scale, nblocks, v_ld);                   \
   }
     const int nk = d / 16, nv = vd / 16;
     if (nk <= 4 && nv <= 4) SA_MFMA(4, 4)
@@ -1282,7 +1284,7 @@ GRAG_API hipError_t grag_sink_attn_prefill(const void* q, const void* k_cache, c
     }
     hipLaunchKernelGGL(sink_attn_prefill_kernel<T>, grid, dim3(256), bytes, st, (const T*)q, (const T*)k_cache,
                        (const T*)v_cache, (T*)out, out_ld, block_tables, bt_stride, q_start, ctx_len, sinks, H, G, d,
-                       vd, BS, scale, out_scale, KT, nblocks);
+                       vd, BS, scale, out_scale, KT, nblocks, v_ld);
   })
   return hipGetLastError();
 }
@@ -1293,10 +1295,10 @@ GRAG_API hipError_t grag_sink_attn_decode(const void* q, const void* k_cache, co
                                           int out_ld, const int* block_tables, int bt_stride, const int* ctx_len,
                                           const float* sinks, int nseq, int H, int G, int d, int vd, int BS,
                                           float scale, float out_scale, int nblocks, int dt, int nsplit,
-                                          int split_len, float* part_o, float* part_ml, hipStream_t st) {
+                                          int split_len, float* part_o, float* part_ml, int v_ld, hipStream_t st) {
   if (nseq <= 0) return hipSuccess;
-  if (vd > 64 * SA_VC || G <= 0 || H % G) return hipErrorInvalidValue;
-  if (dt == 0 && d % 16 == 0 && vd % 16 == 0 && d <= 256 && vd <= 256 && G * ((H / G + 15) / 16) <= 65535 &&
+  if (vd > 64 * SA_VC || G <= 0 || H % G || v_ld < vd) return hipErrorInvalidValue;
+  if (dt == 0 && v_ld % 8 == 0 && (reinterpret_cast<uintptr_t>(v_cache) & 15) == 0 && d % 16 == 0 && vd % 16 == 0 && d <= 256 && vd <= 256 && G * ((H / G + 15) / 16) <= 65535 &&
       out_ld % 4 == 0 && (reinterpret_cast<uintptr_t>(out) & 7) == 0 && (reinterpret_cast<uintptr_t>(q) & 7) == 0 &&
       nseq <= 65535) {
     if (nsplit < 1 || part_o == nullptr || part_ml == nullptr || split_len % 64) nsplit = 1;
@@ -1314,7 +1316,7 @@ GRAG_API hipError_t grag_sink_attn_decode(const void* q, const void* k_cache, co
     hipLaunchKernelGGL((sink_attn_decode_mfma_kernel<NK, NV, 0>), mgrid, dim3(256), mb, st, (const bf16*)q,          \
                        (const bf16*)k_cache, (const bf16*)v_cache, (bf16*)out, out_ld, block_tables, bt_stride,      \
                        ctx_len, sinks, H, G, d, vd, BS, scale, out_scale, nblocks, nsplit, split_len, part_o,        \
-                       part_ml, 0, (const bf16*)nullptr, 0);                                                         \
+                       part_ml, 0, (const bf16*)nullptr, 0, v_ld);                                                   \
   }
     const int nk = d / 16, nv = vd / 16;
     if (nk <= 4 && nv <= 4) SD_MFMA(4, 4)
@@ -1329,15 +1331,15 @@ GRAG_API hipError_t grag_sink_attn_decode(const void* q, const void* k_cache, co
     return hipGetLastError();
   }
   const size_t bytes = ((size_t)d + 4 * 64 + 8 + 4 * (size_t)vd) * sizeof(float);
-  if (dt == 0 && d % 8 == 0 && vd % 2 == 0 && vd <= 256) {
+  if (dt == 0 && d % 8 == 0 && vd % 2 == 0 && vd <= 256 && v_ld % 2 == 0 && (reinterpret_cast<uintptr_t>(v_cache) & 3) == 0) {
     hipLaunchKernelGGL(sink_attn_decode_vec_kernel, dim3(H, nseq), dim3(256), bytes, st, (const bf16*)q,
                        (const bf16*)k_cache, (const bf16*)v_cache, (bf16*)out, out_ld, block_tables, bt_stride,
-                       ctx_len, sinks, H, G, d, vd, BS, scale, out_scale, nblocks);
+                       ctx_len, sinks, H, G, d, vd, BS, scale, out_scale, nblocks, v_ld);
     return hipGetLastError();
   }
   DT_DISPATCH(dt, hipLaunchKernelGGL(sink_attn_decode_kernel<T>, dim3(H, nseq), dim3(256), bytes, st, (const T*)q,
                                      (const T*)k_cache, (const T*)v_cache, (T*)out, out_ld, block_tables, bt_stride,
-                                     ctx_len, sinks, H, G, d, vd, BS, scale, out_scale, nblocks);)
+                                     ctx_len, sinks, H, G, d, vd, BS, scale, out_scale, nblocks, v_ld);)
   return hipGetLastError();
 }
 
@@ -1366,7 +1368,7 @@ GRAG_API hipError_t grag_window_decode_mfma(const void* q, const void* k_cache, 
     hipLaunchKernelGGL((sink_attn_decode_mfma_kernel<NK, NV, 1>), mgrid, dim3(256), mb, st, (const bf16*)q,          \
                        (const bf16*)k_cache, (const bf16*)v_cache, (bf16*)out, out_ld, block_tables, bt_stride,      \
                        ctx_len, bias, H, G, d, vd, BS, scale, 1.f, nblocks, 1, 0, (float*)nullptr, (float*)nullptr,  \
-                       window, (const bf16*)gate, gate_ld);                                                          \
+                       window, (const bf16*)gate, gate_ld, vd);                                                      \
   }
   if (d <= 64 && vd <= 64) SW_MFMA(4, 4)
   else SW_MFMA(8, 8)

@@ -215,7 +215,7 @@ def _namudra_kernel_table(dev, H=28, G=4, D=128, W=3584, T=2048, B=64, ctx=2048,
         flops=4.0 * pairs * H * D)
     add("zofesun sink_attn_prefill", _timed(lambda: sink_attention(q, kc, vc, meta, 0.09, pb)), flops=4.0 * T * T / 2 * H * D)
     kl = torch.randn(nb + 1, 1, bs, R + r, device=dev).to(bf)
-    vl = torch.randn(nb + 1, 1, bs, R, device=dev).to(bf)
+    vl = kl[..., :R]
     ql = torch.randn(T, H, R + r, device=dev).to(bf)
     add("latent attention prefill (sink kernel, no sink)", _timed(lambda: sink_attention(ql, kl, vl, meta, 0.06, None)),
         flops=2.0 * T * T / 2 * H * (2 * R + r))
@@ -228,10 +228,10 @@ def _namudra_kernel_table(dev, H=28, G=4, D=128, W=3584, T=2048, B=64, ctx=2048,
         bytes_=2.0 * B * win * G * D * 2)
     add("zofesun sink_attn_decode", _timed(lambda: sink_attention(qd, kd, vd_, dmeta, 0.09, pb)), bytes_=2.0 * B * ctx * G * D * 2)
     kld = torch.randn(B * nbd + 1, 1, bs, R + r, device=dev).to(bf)
-    vld = torch.randn(B * nbd + 1, 1, bs, R, device=dev).to(bf)
+    vld = kld[..., :R]
     qld = torch.randn(B, H, R + r, device=dev).to(bf)
     add("latent attention decode (sink kernel, no sink)", _timed(lambda: sink_attention(qld, kld, vld, dmeta, 0.06, None)),
-        bytes_=B * ctx * (2 * R + r) * 2.0)
+        bytes_=B * ctx * (R + r) * 2.0)
     # ---- projection post-processing + cache stores
     proj = torch.randn(T, (2 * H + G) * D, device=dev).to(bf)
     ones = torch.ones(D, device=dev)
@@ -244,8 +244,8 @@ def _namudra_kernel_table(dev, H=28, G=4, D=128, W=3584, T=2048, B=64, ctx=2048,
     ckv = torch.randn(T, R + r, device=dev).to(bf)
     tabr = rope_table(T, r, 1e4, dev)
     wR, wq4 = torch.ones(R, device=dev), torch.ones(W // 4, device=dev)
-    add("latent_store", _timed(lambda: latent_store(ckv, wR, pos, tabr, meta.slot_mapping, ql, kl, vl, 1e-6)),
-        bytes_=T * ((R + r) * 2 + R + 2 * H * r) * 2.0)
+    add("latent_store", _timed(lambda: latent_store(ckv, wR, pos, tabr, meta.slot_mapping, ql, kl, 1e-6)),
+        bytes_=T * ((R + r) * 2 + 2 * H * r) * 2.0)
     cq = torch.randn(T, 2 * (W // 4), device=dev).to(bf)
     add("rmsnorm_rows (query latent)", _timed(lambda: rmsnorm_rows(cq[:, : W // 4], wq4, 1e-6)),
         bytes_=T * (W // 4) * 2 * 2.0)

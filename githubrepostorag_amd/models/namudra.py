@@ -17,8 +17,9 @@ Mixers:
   "latent_attention"  causal softmax attention over a cached latent plus one rotated key part shared by the heads.
                       The key and value expansions are folded into the query and output projections when the
                       weights are loaded (W_q' = W_uk^T W_uq per head, W_o' = W_o W_uv per head), so a step attends
-                      straight to the cache: one kv head whose key is latent | rotated part and whose value is the
-                      latent                  [grag_rmsnorm_rows, grag_latent_store, grag_sink_attn_* without sink]
+                      straight to the cache: one kv head whose key rows are latent | rotated part and whose value
+                      rows are the head of the same rows  [grag_rmsnorm_rows, grag_latent_store, grag_sink_attn_*
+                                                           without sink]
 
 Per layer the mixer's input projections are one GEMM (q | k | v | g, q | k | g, or dq | dkv), gate and up are one
 GEMM, and every sublayer boundary is one kernel: streams update, next read-out, next norm [grag_hyper_mix].
@@ -232,36 +233,37 @@ class NamudraModel:
         return n
 
     # ------------------------------------------------------------------ cache and state
-    def _kv_shape(self, li: int):
-        """(key row, value row) sizes per cached token of a layer, kv heads; None for layers without a cache."""
-        L = self.cfg.layers[li].mixer
-        a = L.spec
-        if L.kind == "attention":
-            return a.kv_heads, a.dim, a.dim
-        if L.kind == "latent_attention":
-            return 1, a.kv_rank + a.rot_dim, a.kv_rank
-        return None
+    def _kv_row(self, li: int) -> int:
+        """Numbers cached per token by a layer (0: no cache)."""
+        m = self.cfg.layers[li].mixer
+        if m.kind == "attention":
+            return 2 * m.spec.kv_heads * m.spec.dim
+        if m.kind == "latent_attention":
+            return m.spec.kv_rank + m.spec.rot_dim
+        return 0
 
     def kv_bytes_per_block(self, block_size: int) -> int:
-        n = 0
-        for li, _, _ in self.runs:
-            s = self._kv_shape(li)
-            if s is not None:
-                n += s[0] * block_size * (s[1] + s[2])
+        n = sum(self._kv_row(li) for li, _, _ in self.runs) * block_size
         return max(1, n) * torch.finfo(self.dtype).bits // 8
 
     def allocate_kv_cache(self, num_blocks: int, block_size: int):
-        """One (K [blocks, G, BS, key], V [blocks, G, BS, value]) pair per run of a layer with attention (None for
-        retention runs); a looped layer has one pair per pass.  Windowed layers: normed keys | keys as projected;
-        latent layers: (latent | rotated part) | latent, one head."""
+        """One (K, V) pair per run of a layer with attention (None for retention runs); a looped layer has one pair
+        per pass.  Windowed layers: normed keys [blocks, G, BS, dim] and keys as projected, the values, in a
+        tensor of their own.  Latent layers: one tensor [blocks, 1, BS, kv_rank + rot_dim] (latent | rotated part);
+        its values are the latents, so V is a view of the first kv_rank columns of the same rows."""
         caches = []
         for li, _, _ in self.runs:
-            s = self._kv_shape(li)
-            if s is None:
+            m = self.cfg.layers[li].mixer
+            a = m.spec
+            z = dict(dtype=self.dtype, device=self.device)
+            if m.kind == "attention":
+                caches.append((torch.zeros(num_blocks, a.kv_heads, block_size, a.dim, **z),
+                               torch.zeros(num_blocks, a.kv_heads, block_size, a.dim, **z)))
+            elif m.kind == "latent_attention":
+                k = torch.zeros(num_blocks, 1, block_size, a.kv_rank + a.rot_dim, **z)
+                caches.append((k, k[..., : a.kv_rank]))
+            else:
                 caches.append(None)
-                continue
-            caches.append(tuple(torch.zeros(num_blocks, s[0], block_size, n, dtype=self.dtype, device=self.device)
-                                for n in s[1:]))
         return caches
 
     def state_bytes_per_slot(self) -> int:
@@ -304,7 +306,7 @@ class NamudraModel:
         qr = L.off[1]
         cq = rmsnorm_rows(p[:, :qr], L.dqn, eps)
         q = linear(cq, L.wq).view(T, a.heads, a.kv_rank + a.rot_dim)
-        latent_store(p[:, qr:], L.ckn, positions, self._tables[L.rope], meta.slot_mapping, q, kc, vc, eps)
+        latent_store(p[:, qr:], L.ckn, positions, self._tables[L.rope], meta.slot_mapping, q, kc, eps)
         return linear(sink_attention(q, kc, vc, meta, a.scale, None), L.wo)
 
     def forward(self, input_ids: torch.Tensor, positions: torch.Tensor, meta: AttnMetadata, kv_caches,

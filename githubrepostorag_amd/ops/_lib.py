@@ -82,8 +82,8 @@ _SIGS = {
     "grag_embed_f32": [P, P, P, I, I, I, I, P],
     "grag_dyt_residual": [P, F, P, P, P, P, P, F, P, P, P, I, I, I, P],
     "grag_rope_vnorm_store": [P, I, I, I, I, P, P, I, P, P, P, P, I, I, I, I, I, I, I, ctypes.c_long, F, I, P],
-    "grag_sink_attn_prefill": [P, P, P, P, I, P, I, P, P, P, I, I, I, I, I, I, I, F, F, I, I, P],
-    "grag_sink_attn_decode": [P, P, P, P, I, P, I, P, P, I, I, I, I, I, I, F, F, I, I, I, I, P, P, P],
+    "grag_sink_attn_prefill": [P, P, P, P, I, P, I, P, P, P, I, I, I, I, I, I, I, F, F, I, I, I, P],
+    "grag_sink_attn_decode": [P, P, P, P, I, P, I, P, P, I, I, I, I, I, I, F, F, I, I, I, I, P, P, I, P],
     "grag_decay_attn_scan": [P, I, I, I, I, P, P, P, P, P, P, I, I, I, I, I, I, P, I, I, P, P, I, I, F, P],
     "grag_decay_attn_chunk": [],
     "grag_mingru_chunk": [],
@@ -93,7 +93,7 @@ _SIGS = {
     "grag_hyper_max_streams": [],
     "grag_hyper_mix": [P, I, P, P, P, P, P, F, P, P, I, I, I, P],
     "grag_qk_norm_store": [P, I, I, I, P, P, P, P, P, P, I, I, I, I, I, ctypes.c_long, F, I, P],
-    "grag_latent_store": [P, I, P, P, P, I, P, P, P, P, I, I, I, I, I, ctypes.c_long, F, I, P],
+    "grag_latent_store": [P, I, P, P, P, I, P, P, P, I, I, I, I, I, ctypes.c_long, F, I, P],
     "grag_sigmoid_window_prefill": [P, P, P, P, I, P, I, P, P, P, I, I, I, I, I, I, I, F, I, I, I, P, I, P],
     "grag_sigmoid_window_decode": [P, P, P, P, I, P, I, P, P, I, I, I, I, I, I, F, I, I, I, P, I, P],
     "grag_rmsnorm_rows": [P, I, P, P, I, I, F, I, P],

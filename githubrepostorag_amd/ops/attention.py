@@ -477,7 +477,11 @@ def sink_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
     if not q.is_cuda:
         out.copy_((sink_attention_ref(q, k_cache, v_cache, meta, scale, sinks) * out_scale).reshape(T, H * vd))
         return out
-    assert q.is_contiguous() and out.stride(1) == 1 and sinks.dtype == torch.float32
+    assert q.is_contiguous() and out.stride(1) == 1 and sinks.dtype == torch.float32 and k_cache.is_contiguous()
+    # value rows may be the head of wider rows (a view [..., :vd] of a cache whose rows hold more: latent attention
+    # reads its values out of its key rows): v_ld is the row stride, the block / head strides must follow from it
+    v_ld = v_cache.stride(2)
+    assert v_cache.stride(3) == 1 and v_cache.stride(1) == BS * v_ld and v_cache.stride(0) == G * BS * v_ld
     dt = 0 if q.dtype == torch.bfloat16 else 1
     if meta.is_decode and meta.max_q_len == 1:
         # key splits (flash-decoding) when the step brings a plan and scratch that holds it
@@ -489,11 +493,11 @@ def sink_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
         call("grag_sink_attn_decode", ptr(q), ptr(k_cache), ptr(v_cache), ptr(out), out.stride(0),
              ptr(meta.block_tables), meta.block_tables.stride(0), ptr(meta.ctx_len), ptr(sinks), meta.num_seqs, H, G,
              d, vd, BS, float(scale), float(out_scale), k_cache.shape[0], dt, nsplit, meta.split_len if nsplit > 1 else 0,
-             ptr(meta.part_o) if nsplit > 1 else None, ptr(meta.part_ml) if nsplit > 1 else None)
+             ptr(meta.part_o) if nsplit > 1 else None, ptr(meta.part_ml) if nsplit > 1 else None, v_ld)
     else:
         call("grag_sink_attn_prefill", ptr(q), ptr(k_cache), ptr(v_cache), ptr(out), out.stride(0),
              ptr(meta.block_tables), meta.block_tables.stride(0), ptr(meta.q_start), ptr(meta.ctx_len), ptr(sinks),
-             meta.num_seqs, meta.max_q_len, H, G, d, vd, BS, float(scale), float(out_scale), k_cache.shape[0], dt)
+             meta.num_seqs, meta.max_q_len, H, G, d, vd, BS, float(scale), float(out_scale), k_cache.shape[0], dt, v_ld)
     return out
 
 

@@ -240,15 +240,14 @@ def qk_norm_store(proj: torch.Tensor, qoff: int, koff: int, qw: torch.Tensor, kw
 
 
 def latent_store(ckv: torch.Tensor, cw: torch.Tensor, positions: torch.Tensor, table: torch.Tensor,
-                 slot_mapping: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
-                 eps: float) -> torch.Tensor:
+                 slot_mapping: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, eps: float) -> torch.Tensor:
     """Latent attention's cache row and query rotation.  ``ckv`` [T, R + r]: a latent of R columns and r columns of
-    the key part that all heads share.  Stores latent / rms(latent) * cw | rotated part into k_cache
-    [blocks, 1, BS, R + r] and the normed latent again into v_cache [blocks, 1, BS, R] at ``slot_mapping``;
-    rotates the last r columns of every head of ``q`` [T, H, R + r] in place (``table``: rope_table of width r)."""
+    the key part that all heads share (r = the width of ``table``, a rope_table).  Stores latent / rms(latent) * cw |
+    rotated part into k_cache [blocks, 1, BS, R + r] at ``slot_mapping`` (the attention reads its values, the normed
+    latent, out of the same rows); rotates the last r columns of every head of ``q`` [T, H, R + r] in place."""
     T, H = q.shape[0], q.shape[1]
-    R, BS = v_cache.shape[3], k_cache.shape[2]
-    r = k_cache.shape[3] - R
+    BS, r = k_cache.shape[2], table.shape[1]
+    R = k_cache.shape[3] - r
     if not ckv.is_cuda:
         x = ckv.float()
         c = x[:, :R]
@@ -266,12 +265,11 @@ def latent_store(ckv: torch.Tensor, cw: torch.Tensor, positions: torch.Tensor, t
         ok = slot_mapping >= 0
         sl = slot_mapping[ok].long()
         k_cache[sl // BS, 0, sl % BS] = torch.cat([c, kr], -1)[ok].to(k_cache.dtype)
-        v_cache[sl // BS, 0, sl % BS] = c[ok].to(v_cache.dtype)
         return q
     assert ckv.stride(1) == 1 and q.is_contiguous() and q.shape[2] == R + r and ckv.shape[1] == R + r
-    assert k_cache.dtype == ckv.dtype and v_cache.dtype == ckv.dtype and q.dtype == ckv.dtype
-    assert k_cache.shape[1] == 1 and v_cache.shape[1] == 1 and table.shape[1] == r and cw.numel() == R
+    assert k_cache.dtype == ckv.dtype and q.dtype == ckv.dtype and k_cache.is_contiguous()
+    assert k_cache.shape[1] == 1 and cw.numel() == R and R > 0
     call("grag_latent_store", ptr(ckv), ckv.stride(0), ptr(cw), ptr(positions), ptr(table), table.shape[0],
-         ptr(slot_mapping), ptr(q), ptr(k_cache), ptr(v_cache), T, H, R, r, BS, k_cache.shape[0] * BS, float(eps),
+         ptr(slot_mapping), ptr(q), ptr(k_cache), T, H, R, r, BS, k_cache.shape[0] * BS, float(eps),
          0 if ckv.dtype == torch.bfloat16 else 1)
     return q

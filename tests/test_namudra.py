@@ -273,7 +273,7 @@ def latent_case(device, dtype, tol):
     wq = torch.cat([torch.einsum("hdr,hdq->hrq", uk, uq[:, :d]), uq[:, d:]], 1).reshape(H * (R + r), Q)
     dev = torch.device(device)
     kc = torch.zeros(10, 1, bs, R + r, dtype=dtype, device=dev)
-    vc = torch.zeros(10, 1, bs, R, dtype=dtype, device=dev)
+    vc = kc[..., :R]  # the values are the latents: the head of the same rows
     table = rope_table(128, r, 20.0, dev)
     f32 = lambda t: t.float().to(dev)
     got = []
@@ -283,7 +283,7 @@ def latent_case(device, dtype, tol):
         cq = rmsnorm_rows(proj[:, :Q], f32(wt["dq.norm"]), 1e-6)
         q = (cq.double().cpu() @ wq.T).to(dtype).to(dev).view(b - a, H, R + r).contiguous()
         latent_store(proj[:, Q:], f32(wt["dkv.norm"]), torch.arange(a, b, dtype=torch.int32, device=dev), table,
-                     meta.slot_mapping, q, kc, vc, 1e-6)
+                     meta.slot_mapping, q, kc, 1e-6)
         o = sink_attention(q, kc, vc, meta, 0.9, None).double().cpu().view(b - a, H, R)
         got.append(torch.einsum("thr,hvr->thv", o, uv).reshape(b - a, H * vd))
     assert float((torch.cat(got) - want).abs().max()) < tol
