@@ -97,6 +97,7 @@ _SIGS = {
     "grag_sigmoid_window_prefill": [P, P, P, P, I, P, I, P, P, P, I, I, I, I, I, I, I, F, I, I, I, P, I, P],
     "grag_sigmoid_window_decode": [P, P, P, P, I, P, I, P, P, I, I, I, I, I, I, F, I, I, I, P, I, P],
     "grag_rmsnorm_rows": [P, I, P, P, I, I, F, I, P],
+    "grag_window_decode_mfma": [P, P, P, P, I, P, I, P, P, I, I, I, I, I, I, F, I, I, P, I, P],
     "grag_attn_decode_xcd": [I],
 }
 
